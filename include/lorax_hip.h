@@ -1,0 +1,138 @@
+/*
+ * lorax_hip.h - C ABI of liblorax_hip.so, the gfx950 (MI355X) implementation of the
+ * multi-adapter LoRA hot path of predibase/lorax (BGMV decode, SGMV prefill).
+ *
+ * Every entry point replaces one function of the reference's pybind module
+ * `punica_kernels` (server/punica_kernels/punica_kernels/punica_ops.cc:446-459).
+ * All pointers are device pointers in the current HIP device's memory unless the
+ * comment says otherwise.  `stream` is a hipStream_t passed as void* (NULL = the
+ * default stream).  No entry point allocates, frees or synchronises; every one is
+ * safe to call while `stream` is being captured into a HIP graph.
+ *
+ * Return value: 0 on success, a LORAX_E* code otherwise; the message for the last
+ * failure on the calling thread is returned by lorax_last_error().  Errors are
+ * reported synchronously from host-side argument validation and from the launch
+ * call itself, never later.
+ *
+ * Element types: x, y, v and all weights share one 16-bit float type (`dtype`);
+ * accumulation is fp32.  Rounding points follow the reference's BGMV kernels
+ * (bgmv_impl.cuh:141,189-190) and its per-adapter fallback loop
+ * (lorax_server/utils/layers.py:206-210,190): the fp32 dot product is rounded to
+ * `dtype`, then added to the destination in fp32 and rounded again.
+ */
+#ifndef LORAX_HIP_H
+#define LORAX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LORAX_OK 0
+#define LORAX_EINVAL 1     /* bad argument (null pointer, negative size, bad dtype)         */
+#define LORAX_ENOKERNEL 2  /* shape outside what the kernels cover ("No suitable kernel.") */
+#define LORAX_ELAUNCH 3    /* the HIP runtime refused the launch                            */
+#define LORAX_ETMPSIZE 4   /* tmp buffer size does not match the reference's contract       */
+
+#define LORAX_F16 0
+#define LORAX_BF16 1
+
+/* A layouts accepted by lorax_sgmv_shrink (one adapter's stack, row-major):
+ *   LORAX_A_RH: [num_layers, r, h_in]  - what the reference's custom sgmv_shrink reads
+ *                                        (sgmv_flashinfer.cuh:13-353; ranks 16..128)
+ *   LORAX_A_HR: [num_layers, h_in, r]  - what its cutlass grouped GEMM reads
+ *                                        (sgmv_cutlass.cuh:46; rank 8)               */
+#define LORAX_A_RH 0
+#define LORAX_A_HR 1
+
+/* Size in bytes of the shrink scratch the reference API passes around
+ * (lorax_server/utils/punica.py:145-147; checked at punica_ops.cc:389-390). */
+#define LORAX_SHRINK_TMP_BYTES (8 * 1024 * 1024)
+
+/*
+ * BGMV, both directions.  Replaces dispatch_bgmv (punica_ops.cc:291-334) and the
+ * kernels behind it (bgmv/bgmv_impl.cuh:15-285).
+ *
+ *   for every token b in [0, num_tokens) with idx = indices[b] >= 0:
+ *     W = (dtype*)w_ptrs[idx] + layer_idx * h_out * h_in          // [h_out, h_in]
+ *     y[b * y_stride + y_offset + j] += dtype(scale * sum_k W[j, k] * x[b * h_in + k])
+ *   tokens with indices[b] < 0 are not touched and w_ptrs is not read for them.
+ *
+ * h_in < h_out selects "expand" (h_in is the LoRA rank), otherwise "shrink"
+ * (h_out is the rank), as bgmv_impl.cuh:204.  The rank must be a multiple of 8 in
+ * [8, 128]; the wide dimension a multiple of 8 below 65536 (punica_ops.cc:310).
+ * The reference binds y_offset = 0 and y_stride = h_out (punica_ops.cc:318); other
+ * values let a caller write one projection's slice of a fused q/k/v or gate/up
+ * output in place.
+ */
+int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* indices,
+               int64_t num_tokens, int32_t h_in, int32_t h_out, int64_t y_offset,
+               int64_t y_stride, int64_t layer_idx, float scale, int32_t dtype, void* stream);
+
+/*
+ * SGMV shrink.  Replaces sgmv_shrink (punica_ops.cc:369-411,
+ * sgmv_flashinfer/sgmv_all.cu:10-65) for a_layout = LORAX_A_RH and the shrink
+ * direction of sgmv_cutlass (punica_ops.cc:338-367, sgmv/sgmv_cutlass.cuh:132-178)
+ * for a_layout = LORAX_A_HR.
+ *
+ *   for every segment i in [0, num_segments) with s_end[i] > s_start[i]:
+ *     A = (dtype*)w_ptrs[i] + layer_idx * r * h_in
+ *     v[s_start[i]:s_end[i], :] += dtype(x[s_start[i]:s_end[i], :] @ A_as_[h_in, r])
+ *   empty or negative segments are skipped without reading w_ptrs[i]
+ *   (sgmv_cutlass.cuh:39-44).  Rows at or beyond num_tokens are never accessed.
+ *
+ * r must be a multiple of 16 in [16, 128] for LORAX_A_RH and 8 or a multiple of 16
+ * up to 128 for LORAX_A_HR; h_in a multiple of 8.  `tmp`/`tmp_bytes` is the caller's
+ * scratch and is only validated for presence; the split-K partial sums live in the
+ * library's own per-device workspace (see lorax_init).
+ */
+int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
+                      const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
+                      int32_t h_in, int32_t r, int32_t a_layout, int64_t layer_idx, void* tmp,
+                      int64_t tmp_bytes, int32_t dtype, void* stream);
+
+/*
+ * SGMV expand.  Replaces the expand direction of sgmv_cutlass (punica_ops.cc:338-367,
+ * sgmv/sgmv_cutlass.cuh:86-131).
+ *
+ *   for every segment i with s_end[i] > s_start[i]:
+ *     B = (dtype*)w_ptrs[i] + layer_idx * r * h_out                  // [r, h_out]
+ *     y[s:e, y_offset : y_offset + h_out] += dtype(v[s:e, :] @ B)    // row pitch y_stride
+ *
+ * r must be a multiple of 8 in [8, 128]; h_out, y_offset and y_stride multiples of 8.
+ */
+int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
+                      const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
+                      int32_t h_out, int64_t y_offset, int64_t y_stride, int64_t layer_idx,
+                      void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
+
+/* Bytes of grouped-GEMM argument scratch for `num_problems` segments.  Replaces
+ * sgmv_tmp_size (sgmv/sgmv_cutlass.cuh:54-58): 3 pointers + 3 int64 + one
+ * 3 x int32 problem size per segment = 60 * num_problems. */
+size_t lorax_sgmv_tmp_size(int32_t num_problems);
+
+/*
+ * Allocates (once per device, idempotent) the library's workspace on `device`:
+ * split-K partial sums and their arrival counters.  Call it outside graph capture
+ * before the first SGMV shrink on a device; the reference has no counterpart because
+ * its scratch arrives through `tmp` (punica.py:145-167).  Calls that use the
+ * workspace concurrently on different streams of one device race.
+ */
+int lorax_init(int32_t device);
+
+/* Workspace bytes lorax_init reserves per device. */
+size_t lorax_workspace_bytes(void);
+
+/* Message of the last error on this thread ("" if none).  Host pointer, valid until
+ * the next failing call on the same thread. */
+const char* lorax_last_error(void);
+
+/* Library version string (host pointer, static). */
+const char* lorax_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LORAX_HIP_H */

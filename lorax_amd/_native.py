@@ -1,0 +1,244 @@
+"""ctypes binding of liblorax_hip.so with the call signatures of the reference's pybind
+module ``punica_kernels`` (server/punica_kernels/punica_kernels/punica_ops.cc:446-459):
+``dispatch_bgmv``, ``sgmv_cutlass``, ``sgmv_shrink`` and ``sgmv_cutlass_tmp_size``.
+
+The functions take torch tensors, perform the checks the reference performs with
+TORCH_CHECK (punica_ops.cc:36-43, 291-411) and raise ``RuntimeError`` on any failure.
+There is no other implementation behind them: if the shared library is missing every
+call raises.
+"""
+
+import ctypes
+import os
+from pathlib import Path
+from typing import Optional
+
+import torch  # noqa: F401  (must be imported first so that its HIP runtime is the one in the process)
+
+LIB_PATH = Path(__file__).resolve().parent / "liblorax_hip.so"
+
+F16, BF16 = 0, 1
+A_RH, A_HR = 0, 1
+SHRINK_TMP_BYTES = 8 * 1024 * 1024
+
+_c = ctypes
+_SIGNATURES = {
+    "lorax_bgmv": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int32, _c.c_int32,
+         _c.c_int64, _c.c_int64, _c.c_int64, _c.c_float, _c.c_int32, _c.c_void_p],
+    ),
+    "lorax_sgmv_shrink": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
+         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_void_p, _c.c_int64, _c.c_int32,
+         _c.c_void_p],
+    ),
+    "lorax_sgmv_expand": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
+         _c.c_int32, _c.c_int32, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
+         _c.c_int32, _c.c_void_p],
+    ),
+    "lorax_sgmv_tmp_size": (_c.c_size_t, [_c.c_int32]),
+    "lorax_init": (_c.c_int, [_c.c_int32]),
+    "lorax_workspace_bytes": (_c.c_size_t, []),
+    "lorax_last_error": (_c.c_char_p, []),
+    "lorax_version": (_c.c_char_p, []),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib: Optional[ctypes.CDLL] = None
+_load_error: Optional[str] = None
+_initialised_devices = set()
+
+
+def _load() -> Optional[ctypes.CDLL]:
+    global _lib, _load_error
+    if _lib is not None or _load_error is not None:
+        return _lib
+    path = os.environ.get("LORAX_HIP_LIBRARY", str(LIB_PATH))
+    try:
+        lib = ctypes.CDLL(path)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    except (OSError, AttributeError) as exc:
+        _load_error = f"{path}: {exc}"
+    return _lib
+
+
+def available() -> bool:
+    """True iff liblorax_hip.so is loaded with every expected symbol."""
+    return _load() is not None
+
+
+def load_error() -> Optional[str]:
+    _load()
+    return _load_error
+
+
+def lib() -> ctypes.CDLL:
+    handle = _load()
+    if handle is None:
+        raise RuntimeError(
+            f"liblorax_hip.so is not available ({_load_error}); build it with `python -m lorax_amd.build`. "
+            "There is no non-HIP implementation of the LoRA kernels in this package."
+        )
+    return handle
+
+
+def version() -> str:
+    return lib().lorax_version().decode()
+
+
+def _raise_last(rc: int):
+    msg = lib().lorax_last_error().decode() or f"error code {rc}"
+    raise RuntimeError(msg)
+
+
+def init(device) -> None:
+    """Allocates the library's workspace on `device` (idempotent). Must not run under graph capture."""
+    index = torch.device(device).index
+    if index is None:
+        index = torch.cuda.current_device()
+    if index in _initialised_devices:
+        return
+    rc = lib().lorax_init(index)
+    if rc != 0:
+        _raise_last(rc)
+    _initialised_devices.add(index)
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float16:
+        return F16
+    if t.dtype == torch.bfloat16:
+        return BF16
+    return -1
+
+
+def _check_input(t: torch.Tensor, name: str, dim: int) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dim() != dim:
+        raise RuntimeError(f"{name} must be a {dim}D tensor")
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _check_same(y: torch.Tensor, x: torch.Tensor, *rest: torch.Tensor) -> None:
+    if y.dtype != x.dtype:
+        raise RuntimeError(f"y and x must share one dtype, got {y.dtype} and {x.dtype}")
+    for t in rest:
+        if t.device != x.device:
+            raise RuntimeError(f"all tensors must be on one device, got {t.device} and {x.device}")
+    if y.device != x.device:
+        raise RuntimeError(f"all tensors must be on one device, got {y.device} and {x.device}")
+
+
+def sgmv_cutlass_tmp_size(num_problems: int) -> int:
+    """sgmv_tmp_size, sgmv/sgmv_cutlass.cuh:54-58."""
+    return int(lib().lorax_sgmv_tmp_size(int(num_problems)))
+
+
+def bgmv(y, x, w_ptr, indicies, layer_idx, scale, y_offset=0, y_slice_size=None) -> None:
+    """lorax_bgmv with an optional column window [y_offset, y_offset + y_slice_size) of y."""
+    _check_input(y, "y", 2)
+    _check_input(x, "x", 2)
+    _check_input(w_ptr, "w_ptr", 1)
+    _check_input(indicies, "indicies", 1)
+    _check_same(y, x, w_ptr, indicies)
+    if w_ptr.dtype != torch.int64 or indicies.dtype != torch.int64:
+        raise RuntimeError("w_ptr and indicies must be int64 tensors")
+    if indicies.size(0) != x.size(0):
+        raise RuntimeError(f"CHECK_EQ(indicies.size(0), x.size(0)) failed. {indicies.size(0)} vs {x.size(0)}")
+    if y.size(0) != x.size(0):
+        raise RuntimeError(f"CHECK_EQ(y.size(0), x.size(0)) failed. {y.size(0)} vs {x.size(0)}")
+    h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
+    with torch.cuda.device(x.device):
+        rc = lib().lorax_bgmv(
+            y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), indicies.data_ptr(), x.size(0), x.size(1), h_out,
+            int(y_offset), y.size(1), int(layer_idx), float(scale), _dtype_code(x), _stream(x),
+        )
+    if rc != 0:
+        _raise_last(rc)
+
+
+def dispatch_bgmv(y, x, w_ptr, indicies, layer_idx, scale) -> None:
+    """dispatch_bgmv, punica_ops.cc:291-334."""
+    bgmv(y, x, w_ptr, indicies, layer_idx, scale)
+
+
+def _check_sgmv(y, x, w_ptr, s_start, s_end, tmp) -> None:
+    _check_input(y, "y", 2)
+    _check_input(x, "x", 2)
+    _check_input(w_ptr, "w_ptr", 1)
+    _check_input(s_start, "s_start", 1)
+    _check_input(s_end, "s_end", 1)
+    _check_input(tmp, "tmp", 1)
+    _check_same(y, x, w_ptr, s_start, s_end, tmp)
+    if w_ptr.dtype != torch.int64:
+        raise RuntimeError("w_ptr must be an int64 tensor")
+    if s_start.dtype != torch.int32 or s_end.dtype != torch.int32:
+        raise RuntimeError("s_start and s_end must be int32 tensors")
+    if not (w_ptr.size(0) == s_start.size(0) == s_end.size(0)):
+        raise RuntimeError(
+            f"w_ptr, s_start and s_end must have one entry per segment, got {w_ptr.size(0)}, "
+            f"{s_start.size(0)}, {s_end.size(0)}"
+        )
+    if y.size(0) != x.size(0):
+        raise RuntimeError(f"CHECK_EQ(y.size(0), x.size(0)) failed. {y.size(0)} vs {x.size(0)}")
+
+
+def sgmv_expand(y, x, w_ptr, s_start, s_end, tmp, layer_idx, y_offset=0, y_slice_size=None) -> None:
+    """lorax_sgmv_expand with an optional column window of y."""
+    _check_sgmv(y, x, w_ptr, s_start, s_end, tmp)
+    h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
+    with torch.cuda.device(x.device):
+        rc = lib().lorax_sgmv_expand(
+            y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0),
+            x.size(0), x.size(1), h_out, int(y_offset), y.size(1), int(layer_idx), tmp.data_ptr(),
+            tmp.numel() * tmp.element_size(), _dtype_code(x), _stream(x),
+        )
+    if rc != 0:
+        _raise_last(rc)
+
+
+def _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, a_layout) -> None:
+    _check_sgmv(y, x, w_ptr, s_start, s_end, tmp)
+    if not torch.cuda.is_current_stream_capturing():
+        init(x.device)
+    with torch.cuda.device(x.device):
+        rc = lib().lorax_sgmv_shrink(
+            y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0),
+            x.size(0), x.size(1), y.size(1), a_layout, int(layer_idx), tmp.data_ptr(),
+            tmp.numel() * tmp.element_size(), _dtype_code(x), _stream(x),
+        )
+    if rc != 0:
+        _raise_last(rc)
+
+
+def sgmv_cutlass(y, x, w_ptr, s_start, s_end, tmp, layer_idx) -> None:
+    """dispatch_sgmv_cutlass, punica_ops.cc:338-367: weights are [L, d_in, d_out]; d_in < d_out is the
+    expand configuration, anything else the shrink one (sgmv_cutlass.cuh:86,132)."""
+    if isinstance(x, torch.Tensor) and isinstance(y, torch.Tensor) and x.dim() == 2 and y.dim() == 2:
+        if x.size(1) < y.size(1):
+            return sgmv_expand(y, x, w_ptr, s_start, s_end, tmp, layer_idx)
+    return _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, A_HR)
+
+
+def sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx) -> None:
+    """dispatch_sgmv_shrink, punica_ops.cc:369-411: weights are [L, d_out, d_in], tmp is 8 MiB of uint8."""
+    if isinstance(tmp, torch.Tensor) and tmp.dtype != torch.uint8:
+        raise RuntimeError(f"CHECK_EQ(tmp.scalar_type(), at::ScalarType::Byte) failed. {tmp.dtype}")
+    return _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, A_RH)

@@ -1,0 +1,401 @@
+"""Adapter-side inputs of the LoRA kernels: per-adapter weight stacks and the per-batch
+routing tables (pointer tables, segment bounds, per-token indices) derived from them.
+
+Mirrors, for the LoRA hot path only,
+  * ``lorax_server/adapters/weights.py``: ``AdapterBatchMetadata`` (:15-32),
+    ``LayerAdapterWeights`` (:66-105), ``AdapterBatchData`` (:108-171);
+  * ``lorax_server/adapters/lora.py``: ``LoraWeights`` (:87-140), ``RankSegments``
+    (:213-227), ``BatchLoraWeights`` (:230-396), ``get_scaling_factor`` (:399-407).
+Attribute and method names are the reference's, so its LoRA layer code and its tests
+(server/tests/utils/test_lora.py) read the same against either package.
+"""
+
+from abc import ABC, abstractmethod
+from collections import defaultdict
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Set, Tuple, Type
+
+import torch
+
+from lorax_amd.sgmv import (
+    BGMV_MAX_RANK,
+    MAX_RANK_CUSTOM,
+    get_tmp_tensors,
+    orient_for_rank,
+    pad_rank,
+    use_cutlass_shrink,
+)
+
+LORA = "lora"
+LM_HEAD = "lm_head"
+
+# Stands in for "this segment's adapter has no weights for the layer": its address is what
+# the pointer tables hold for such segments (adapters/lora.py:26,283). It is never read.
+EMPTY_TENSOR = torch.tensor([])
+
+
+@dataclass
+class AdapterBatchMetadata:
+    """adapters/weights.py:15-32."""
+
+    adapter_indices: torch.Tensor  # [num_tokens] adapter index of every token
+    adapter_list: List[int]  # [batch_size] adapter index of every request
+    adapter_set: Set[int]  # distinct adapter indices in the batch
+    adapter_segments: torch.Tensor  # [num_segments + 1] token offsets of the runs
+    segment_indices: List[int]  # [num_segments] adapter index of every run
+
+
+class AdapterWeights(ABC):
+    @classmethod
+    @abstractmethod
+    def get_batch_types(cls) -> List[Type["BatchAdapterWeights"]]:
+        ...
+
+    @property
+    def speculative_tokens(self) -> int:
+        return 0
+
+
+class BatchAdapterWeights(ABC):
+    @abstractmethod
+    def has_adapter(self, adapter_index: int) -> bool:
+        ...
+
+    @classmethod
+    @abstractmethod
+    def key(cls) -> str:
+        ...
+
+    @classmethod
+    @abstractmethod
+    def load(cls, adapter_weights, meta, layer_name, prefill, prefill_head_indices):
+        ...
+
+
+@dataclass
+class LoraConfig:
+    """The fields of adapters/lora.py:29-35 that the hot path reads."""
+
+    r: int
+    lora_alpha: int = 1
+    target_modules: Optional[List[str]] = None
+    fan_in_fan_out: bool = False
+    use_rslora: bool = False
+    base_model_name_or_path: str = ""
+
+
+def get_scaling_factor(lora_alpha: int, r: int, uses_rslora: bool = False) -> float:
+    """adapters/lora.py:399-407."""
+    return lora_alpha / (r**0.5) if uses_rslora else lora_alpha / r
+
+
+class LoraWeights(AdapterWeights):
+    """One adapter's A and B for one layer type, stacked over layers (adapters/lora.py:87-140).
+
+    Constructed from per-layer ``A: [h_in, r]`` and ``B: [r, h_out]``.  Two layouts:
+      prefill (SGMV): weights_a = [L, r, h_in] for 16 <= r <= 128, else [L, h_in, r];
+                      weights_b = [L, r, h_out]
+      decode  (BGMV): weights_a_t = [L, r, h_in]; weights_b_t = [L, h_out, r]
+    The reference keeps one layout at a time and re-transposes the whole stack whenever a batch
+    of the other kind arrives (adapters/lora.py:111-140), which also moves the stack to a new
+    address.  Here the second layout is materialised on first use and then both stay resident,
+    so every pointer handed to the kernels stays valid for the adapter's lifetime; with 288 GB
+    of HBM the extra copy of B (and of A below rank 16) is the cheaper side of that trade.
+    """
+
+    def __init__(self, weights_a: List[torch.Tensor], weights_b: List[torch.Tensor], adapter_config: LoraConfig):
+        has_layers = len(weights_a) > 0
+        self.lora_a_r = weights_a[0].size(1) if has_layers else 1
+        self.lora_b_r = weights_b[0].size(0) if has_layers else 1
+        self._use_cutlass_shrink = use_cutlass_shrink(self.lora_a_r)
+        self._weights_a = torch.stack([orient_for_rank(w, w.size(1)).contiguous() for w in weights_a])
+        self._weights_b = torch.stack(list(weights_b))
+        self._weights_a_t: Optional[torch.Tensor] = None
+        self._weights_b_t: Optional[torch.Tensor] = None
+        self.adapter_config = adapter_config
+
+    @property
+    def weights_a(self) -> torch.Tensor:
+        return self._weights_a
+
+    @property
+    def weights_b(self) -> torch.Tensor:
+        return self._weights_b
+
+    @property
+    def weights_a_t(self) -> torch.Tensor:
+        if self._weights_a_t is None:
+            # only below rank 16 do the two layouts disagree about A
+            a = self._weights_a
+            self._weights_a_t = a.transpose(1, 2).contiguous() if self._use_cutlass_shrink else a
+        return self._weights_a_t
+
+    @property
+    def weights_b_t(self) -> torch.Tensor:
+        if self._weights_b_t is None:
+            self._weights_b_t = self._weights_b.transpose(1, 2).contiguous()
+        return self._weights_b_t
+
+    @classmethod
+    def get_batch_types(cls) -> List[Type[BatchAdapterWeights]]:
+        return [BatchLoraWeights]
+
+    @classmethod
+    def from_peft(
+        cls,
+        lora_A: List[torch.Tensor],
+        lora_B: List[torch.Tensor],
+        config: LoraConfig,
+        world_size: int = 1,
+    ) -> "LoraWeights":
+        """Per-layer PEFT tensors (lora_A.weight [r, h_in], lora_B.weight [h_out, r]) to a stack:
+        transpose, fold alpha/r into B, pad the rank (adapters/lora.py:184-210)."""
+        scale = get_scaling_factor(config.lora_alpha, config.r, config.use_rslora)
+        a_list = [pad_rank(a.transpose(0, 1), dim=1, world_size=world_size) for a in lora_A]
+        b_list = [pad_rank(b.transpose(0, 1) * scale, dim=0, world_size=world_size) for b in lora_B]
+        if a_list:
+            config.r = a_list[0].size(1)
+        return cls(a_list, b_list, config)
+
+
+@dataclass
+class RankSegments:
+    """Kernel arguments of one rank group (adapters/lora.py:213-227)."""
+
+    rank: int
+    lora_a_ptr: torch.Tensor
+    lora_b_ptr: torch.Tensor
+    # prefill (SGMV)
+    tmp_shrink: Optional[torch.Tensor]
+    tmp_expand: Optional[torch.Tensor]
+    segment_starts: Optional[torch.Tensor]
+    segment_ends: Optional[torch.Tensor]
+    # decode (BGMV)
+    indices: Optional[torch.Tensor]
+
+
+def _unwrap(weights):
+    return weights.lora_weights if hasattr(weights, "lora_weights") else weights
+
+
+@dataclass
+class BatchLoraWeights(BatchAdapterWeights):
+    """adapters/lora.py:230-396."""
+
+    lora_a: Dict[int, torch.Tensor]
+    lora_b: Dict[int, torch.Tensor]
+    adapter_index_configs: Dict[int, LoraConfig]
+    rank_data: Dict[int, RankSegments]
+    use_sgmv: bool
+    layer_name: str
+    prefill_head_indices: Optional[torch.Tensor]
+
+    def has_adapter(self, adapter_index: int) -> bool:
+        return adapter_index in self.adapter_index_configs
+
+    def can_vectorize(self, pg) -> bool:
+        within = all(rd.rank // pg.size() <= MAX_RANK_CUSTOM for rd in self.rank_data.values())
+        return within and self.layer_name != LM_HEAD
+
+    @classmethod
+    def key(cls) -> str:
+        return LORA
+
+    @classmethod
+    def load(
+        cls,
+        adapter_weights: Dict[int, AdapterWeights],
+        meta: AdapterBatchMetadata,
+        layer_name: str,
+        prefill: bool,
+        prefill_head_indices: Optional[torch.Tensor],
+    ) -> Optional["BatchLoraWeights"]:
+        loras: Dict[int, LoraWeights] = {}
+        for idx, w in adapter_weights.items():
+            w = _unwrap(w)
+            if isinstance(w, LoraWeights):
+                loras[idx] = w
+        if not loras:
+            return None
+
+        seg_adapters = list(meta.segment_indices)
+        covered = [s for s, idx in enumerate(seg_adapters) if idx in loras]
+        if not covered:
+            return None
+        device = next(iter(loras.values())).weights_a.device
+
+        lora_a = {seg_adapters[s]: loras[seg_adapters[s]].weights_a for s in covered}
+        lora_b = {seg_adapters[s]: loras[seg_adapters[s]].weights_b for s in covered}
+        max_rank = max(loras[seg_adapters[s]].lora_a_r for s in covered)
+        use_sgmv = bool(prefill or max_rank > BGMV_MAX_RANK)
+
+        # One pointer per segment; segments without weights hold a placeholder address that no
+        # rank group refers to.
+        null = EMPTY_TENSOR.data_ptr()
+        if use_sgmv:
+            a_addr = [loras[i].weights_a.data_ptr() if i in loras else null for i in seg_adapters]
+            b_addr = [loras[i].weights_b.data_ptr() if i in loras else null for i in seg_adapters]
+        else:
+            a_addr = [loras[i].weights_a_t.data_ptr() if i in loras else null for i in seg_adapters]
+            b_addr = [loras[i].weights_b_t.data_ptr() if i in loras else null for i in seg_adapters]
+        lora_a_ptr = torch.tensor(a_addr, dtype=torch.int64, device=device)
+        lora_b_ptr = torch.tensor(b_addr, dtype=torch.int64, device=device)
+
+        configs = {seg_adapters[s]: loras[seg_adapters[s]].adapter_config for s in covered}
+
+        by_rank: Dict[int, List[int]] = defaultdict(list)
+        for s in covered:
+            by_rank[loras[seg_adapters[s]].lora_a_r].append(s)
+
+        head_starts = head_ends = None
+        if prefill_head_indices is not None:
+            # LM-head inputs keep one row per request; recount segment bounds in those rows
+            head_starts, head_ends = [0], [0]
+            bounds = meta.adapter_segments.tolist()
+            j = 1
+            for head_index in prefill_head_indices.tolist():
+                if head_index < bounds[j]:
+                    head_ends[-1] += 1
+                else:
+                    head_starts.append(head_ends[-1])
+                    head_ends.append(head_ends[-1] + 1)
+                    j += 1
+
+        token_adapters = None if use_sgmv else meta.adapter_indices.tolist()
+        rank_data: Dict[int, RankSegments] = {}
+        for rank, segs in by_rank.items():
+            tmp_shrink = tmp_expand = starts = ends = token_slots = None
+            if use_sgmv:
+                tmp_shrink, tmp_expand = get_tmp_tensors(len(segs), rank, device)
+                starts = meta.adapter_segments[segs]
+                ends = meta.adapter_segments[[s + 1 for s in segs]]
+                if head_starts is not None:
+                    for i, s in enumerate(segs):
+                        starts[i] = head_starts[s]
+                        ends[i] = head_ends[s]
+            else:
+                # slot of an adapter = position of its first segment inside this group's pointer slice
+                slot: Dict[int, int] = {}
+                for pos, s in enumerate(segs):
+                    slot.setdefault(seg_adapters[s], pos)
+                token_slots = torch.tensor(
+                    [slot.get(a, -1) if (a in loras and loras[a].lora_a_r == rank) else -1 for a in token_adapters],
+                    dtype=torch.int64,
+                    device=device,
+                )
+            rank_data[rank] = RankSegments(
+                rank=rank,
+                lora_a_ptr=lora_a_ptr[segs],
+                lora_b_ptr=lora_b_ptr[segs],
+                tmp_shrink=tmp_shrink,
+                tmp_expand=tmp_expand,
+                segment_starts=starts,
+                segment_ends=ends,
+                indices=token_slots,
+            )
+
+        return cls(
+            lora_a=lora_a,
+            lora_b=lora_b,
+            adapter_index_configs=configs,
+            rank_data=rank_data,
+            use_sgmv=use_sgmv,
+            layer_name=layer_name,
+            prefill_head_indices=prefill_head_indices,
+        )
+
+
+class LayerAdapterWeights:
+    """All adapters loaded for one layer type (adapters/weights.py:66-105)."""
+
+    def __init__(self):
+        self.adapter_weights: Dict[int, AdapterWeights] = {}
+
+    def add_adapter(self, adapter_idx: int, weights: AdapterWeights):
+        self.adapter_weights[adapter_idx] = weights
+
+    def remove_adapter(self, adapter_idx: int):
+        self.adapter_weights.pop(adapter_idx, None)
+
+    @property
+    def max_speculative_tokens(self) -> int:
+        return max(w.speculative_tokens for w in self.adapter_weights.values())
+
+    def is_empty(self) -> bool:
+        return not self.adapter_weights
+
+    def get_data(
+        self,
+        meta: AdapterBatchMetadata,
+        layer_name: str,
+        prefill: bool,
+        prefill_head_indices: Optional[torch.Tensor],
+    ) -> Dict[str, BatchAdapterWeights]:
+        per_type: Dict[Type[BatchAdapterWeights], Dict[int, AdapterWeights]] = defaultdict(dict)
+        for idx, w in self.adapter_weights.items():
+            for batch_type in w.get_batch_types():
+                per_type[batch_type][idx] = w
+        out = {}
+        for batch_type, group in per_type.items():
+            batched = batch_type.load(group, meta, layer_name, prefill, prefill_head_indices)
+            if batched is not None:
+                out[batch_type.key()] = batched
+        return out
+
+
+@dataclass
+class AdapterBatchData:
+    """adapters/weights.py:108-171. ``punica_wrapper`` and ``layer_to_lora_weights`` belong to the
+    reference's Triton path and are always None/empty here."""
+
+    meta: AdapterBatchMetadata
+    data: Dict[str, Dict[str, BatchAdapterWeights]]  # layer type -> adapter type -> batch data
+    layer_to_lora_weights: Dict[Tuple[str, int], Tuple[torch.Tensor, torch.Tensor]]
+    punica_wrapper: Optional[object]
+    prefill: bool
+
+    @staticmethod
+    def from_meta(
+        meta: AdapterBatchMetadata,
+        weights: Dict[str, LayerAdapterWeights],
+        layer_to_lora_weights: Optional[Dict] = None,
+        punica_wrapper: Optional[object] = None,
+        prefill: bool = False,
+        prefill_head_indices: Optional[torch.Tensor] = None,
+    ) -> "AdapterBatchData":
+        data = {}
+        for layer_name, layer_weights in weights.items():
+            if layer_weights.is_empty():
+                continue
+            head = prefill_head_indices if layer_name == LM_HEAD else None
+            batched = layer_weights.get_data(meta, layer_name, prefill, head)
+            if batched:
+                data[layer_name] = batched
+        return AdapterBatchData(
+            meta=meta,
+            data=data,
+            layer_to_lora_weights=layer_to_lora_weights or {},
+            punica_wrapper=punica_wrapper,
+            prefill=prefill,
+        )
+
+    def ranks(self) -> Set[int]:
+        found = set()
+        for layer_data in self.data.values():
+            lora = layer_data.get(LORA)
+            if lora is not None:
+                found.update(rd.rank for rd in lora.rank_data.values())
+        return found
+
+    def layer_names(self) -> Set[str]:
+        return set(self.data.keys())
+
+    def adapter_keys(self) -> Set[str]:
+        keys = set()
+        for layer_data in self.data.values():
+            keys.update(layer_data.keys())
+        return keys
+
+    @property
+    def max_rank(self) -> int:
+        return max(self.ranks(), default=0)

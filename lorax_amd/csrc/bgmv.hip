@@ -1,0 +1,291 @@
+// BGMV for gfx950: per-token gathered LoRA matrix-vector products for decode batches.
+//
+// Semantics follow the reference kernels in punica_kernels/bgmv/bgmv_impl.cuh:
+//   shrink (:15-143):  v[b, j] += T(scale * sum_k A[idx][layer, j, k] * x[b, k])
+//   expand (:146-192): y[b, j] += T(scale * sum_k B[idx][layer, j, k] * v[b, k])
+// for every token b whose idx = indices[b] is >= 0 (:24-27, :157-159).
+//
+// The reference launches one block per (output element, token) for shrink and one
+// per (32 outputs, token) for expand, so every token re-reads its adapter's weights.
+// Here the tokens of one adapter are grouped inside the kernel (group_tokens) and a
+// workgroup streams the adapter's rows once for up to kGroup tokens, with 16-byte
+// loads, fp32 accumulation in registers and one wave reduction per output.
+#include "kernels.h"
+
+namespace lorax {
+
+constexpr int kBgmvThreads = 256;
+constexpr int kGroup = 4;  // tokens sharing one pass over an adapter's weights
+
+template <int N>
+struct Pow2Ceil {
+  static constexpr int value = N <= 1 ? 1 : 2 * Pow2Ceil<(N + 1) / 2>::value;
+};
+
+// ---------------------------------------------------------------------------------
+// Shrink: rows of A are h_in long (thousands of elements); a workgroup owns RS rows
+// of one adapter and NT tokens and walks the hidden dimension once.
+// ---------------------------------------------------------------------------------
+template <typename D, int RS, int NT>
+__device__ __forceinline__ void bgmv_shrink_body(typename D::E* __restrict__ Y,
+                                                 const typename D::E* __restrict__ X,
+                                                 const typename D::E* __restrict__ A,
+                                                 const int (&toks)[kGroup], int h_in, int row0,
+                                                 int64_t y_offset, int64_t y_stride, float scale,
+                                                 float* red) {
+  using vec8 = typename D::vec8;
+  const int tid = threadIdx.x;
+  float acc[RS][NT];
+#pragma unroll
+  for (int j = 0; j < RS; ++j)
+#pragma unroll
+    for (int g = 0; g < NT; ++g) acc[j][g] = 0.f;
+
+  const typename D::E* xrow[NT];
+#pragma unroll
+  for (int g = 0; g < NT; ++g) xrow[g] = X + static_cast<int64_t>(toks[g]) * h_in;
+
+#pragma unroll 2
+  for (int k = tid * 8; k < h_in; k += kBgmvThreads * 8) {
+    vec8 xv[NT];
+    vec8 wv[RS];
+#pragma unroll
+    for (int g = 0; g < NT; ++g) xv[g] = load8<D>(xrow[g] + k);
+#pragma unroll
+    for (int j = 0; j < RS; ++j) wv[j] = load8<D>(A + static_cast<int64_t>(j) * h_in + k);
+    float xf[NT][8];
+#pragma unroll
+    for (int g = 0; g < NT; ++g)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xf[g][e] = to_f32<D>(xv[g][e]);
+#pragma unroll
+    for (int j = 0; j < RS; ++j) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float w = to_f32<D>(wv[j][e]);
+#pragma unroll
+        for (int g = 0; g < NT; ++g) acc[j][g] = fmaf(w, xf[g][e], acc[j][g]);
+      }
+    }
+  }
+
+  // Wave reduction of the RS*NT sums, then across the four waves through LDS.
+  constexpr int NV = Pow2Ceil<RS * NT>::value;
+  float vals[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) vals[i] = 0.f;
+#pragma unroll
+  for (int j = 0; j < RS; ++j)
+#pragma unroll
+    for (int g = 0; g < NT; ++g) vals[j * NT + g] = acc[j][g];
+  transpose_reduce<NV>(vals);
+  const int lane = lane_id();
+  const int wave = tid / kWave;
+  if ((lane & (kWave / NV - 1)) == 0) red[wave * NV + transpose_reduce_index<NV>(lane)] = vals[0];
+  __syncthreads();
+  if (tid < RS * NT) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < kBgmvThreads / kWave; ++w) s += red[w * NV + tid];
+    const int j = tid / NT;
+    const int g = tid % NT;
+    int tok = toks[0];
+#pragma unroll
+    for (int q = 1; q < NT; ++q)
+      if (g == q) tok = toks[q];
+    typename D::E* yp = Y + static_cast<int64_t>(tok) * y_stride + y_offset + row0 + j;
+    *yp = accumulate<D>(*yp, s * scale);
+  }
+}
+
+template <typename D, int RS>
+__global__ __launch_bounds__(kBgmvThreads) void bgmv_shrink_kernel(
+    typename D::E* __restrict__ Y, const typename D::E* __restrict__ X,
+    const int64_t* __restrict__ W, const int64_t* __restrict__ indices, int num_tokens, int h_in,
+    int r, int64_t y_offset, int64_t y_stride, int64_t layer_idx, float scale) {
+  __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<RS * kGroup>::value];
+  const int b = blockIdx.y;
+  const int64_t idx = indices[b];
+  if (idx < 0) return;
+  int toks[kGroup];
+  const int n = group_tokens<kGroup>(indices, num_tokens, b, idx, toks);
+  if (n == 0) return;
+  const int row0 = blockIdx.x * RS;
+  const typename D::E* A = reinterpret_cast<const typename D::E*>(W[idx]) +
+                           (layer_idx * r + row0) * static_cast<int64_t>(h_in);
+  switch (n) {
+    case 1:
+      bgmv_shrink_body<D, RS, 1>(Y, X, A, toks, h_in, row0, y_offset, y_stride, scale, red);
+      break;
+    case 2:
+      bgmv_shrink_body<D, RS, 2>(Y, X, A, toks, h_in, row0, y_offset, y_stride, scale, red);
+      break;
+    case 3:
+      bgmv_shrink_body<D, RS, 3>(Y, X, A, toks, h_in, row0, y_offset, y_stride, scale, red);
+      break;
+    default:
+      bgmv_shrink_body<D, RS, 4>(Y, X, A, toks, h_in, row0, y_offset, y_stride, scale, red);
+      break;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Expand: rows of B^T are only r long, adjacent output columns are adjacent in memory.
+// CP lanes (a power of two >= r/8) cover one column with one 16-byte load each, so a
+// wave reads a contiguous run of 64/CP columns per step; the CP partial dot products
+// meet in a sub-wave shuffle and the first lane of the group updates y.
+// ---------------------------------------------------------------------------------
+template <typename D, int CP, int U, int NT>
+__device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
+                                                 const typename D::E* __restrict__ V,
+                                                 const typename D::E* __restrict__ B,
+                                                 const int (&toks)[kGroup], int r, int h_out,
+                                                 int col0, int64_t y_offset, int64_t y_stride,
+                                                 float scale) {
+  using vec8 = typename D::vec8;
+  using E = typename D::E;
+  constexpr int kCols = kBgmvThreads / CP;  // columns per step of the workgroup
+  const int tid = threadIdx.x;
+  const int part = tid % CP;
+  const bool has_k = part * 8 < r;
+
+  float vf[NT][8];
+#pragma unroll
+  for (int g = 0; g < NT; ++g) {
+    vec8 vv = zero8<D>();
+    if (has_k) vv = load8<D>(V + static_cast<int64_t>(toks[g]) * r + part * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) vf[g][e] = to_f32<D>(vv[e]);
+  }
+
+  vec8 wv[U];
+  E yv[U][NT];
+  int col[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    col[u] = col0 + u * kCols + tid / CP;
+    wv[u] = zero8<D>();
+    if (has_k && col[u] < h_out) wv[u] = load8<D>(B + static_cast<int64_t>(col[u]) * r + part * 8);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int g = 0; g < NT; ++g) {
+      yv[u][g] = static_cast<E>(0.f);
+      if (part == 0 && col[u] < h_out)
+        yv[u][g] = Y[static_cast<int64_t>(toks[g]) * y_stride + y_offset + col[u]];
+    }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    float s[NT];
+#pragma unroll
+    for (int g = 0; g < NT; ++g) s[g] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float w = to_f32<D>(wv[u][e]);
+#pragma unroll
+      for (int g = 0; g < NT; ++g) s[g] = fmaf(w, vf[g][e], s[g]);
+    }
+#pragma unroll
+    for (int m = CP / 2; m >= 1; m >>= 1)
+#pragma unroll
+      for (int g = 0; g < NT; ++g) s[g] += __shfl_xor(s[g], m, kWave);
+    if (part == 0 && col[u] < h_out) {
+#pragma unroll
+      for (int g = 0; g < NT; ++g)
+        Y[static_cast<int64_t>(toks[g]) * y_stride + y_offset + col[u]] =
+            accumulate<D>(yv[u][g], s[g] * scale);
+    }
+  }
+}
+
+template <typename D, int CP, int U>
+__global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(
+    typename D::E* __restrict__ Y, const typename D::E* __restrict__ V,
+    const int64_t* __restrict__ W, const int64_t* __restrict__ indices, int num_tokens, int r,
+    int h_out, int64_t y_offset, int64_t y_stride, int64_t layer_idx, float scale) {
+  const int b = blockIdx.y;
+  const int64_t idx = indices[b];
+  if (idx < 0) return;
+  int toks[kGroup];
+  const int n = group_tokens<kGroup>(indices, num_tokens, b, idx, toks);
+  if (n == 0) return;
+  const int col0 = blockIdx.x * (kBgmvThreads / CP) * U;
+  const typename D::E* B =
+      reinterpret_cast<const typename D::E*>(W[idx]) + layer_idx * h_out * static_cast<int64_t>(r);
+  switch (n) {
+    case 1:
+      bgmv_expand_body<D, CP, U, 1>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale);
+      break;
+    case 2:
+      bgmv_expand_body<D, CP, U, 2>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale);
+      break;
+    case 3:
+      bgmv_expand_body<D, CP, U, 3>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale);
+      break;
+    default:
+      bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale);
+      break;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Host-side launchers
+// ---------------------------------------------------------------------------------
+template <typename D, int RS>
+static hipError_t launch_shrink_rs(const BgmvArgs& a, hipStream_t stream) {
+  dim3 grid(a.h_out / RS, static_cast<unsigned>(a.num_tokens));
+  hipLaunchKernelGGL((bgmv_shrink_kernel<D, RS>), grid, dim3(kBgmvThreads), 0, stream,
+                     static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x),
+                     a.w_ptrs, a.indices, static_cast<int>(a.num_tokens), a.h_in, a.h_out,
+                     a.y_offset, a.y_stride, a.layer_idx, a.scale);
+  return hipGetLastError();
+}
+
+template <typename D>
+static hipError_t launch_shrink(const BgmvArgs& a, hipStream_t stream) {
+  // Rows per workgroup: 8 when the grid is large enough to fill 256 CUs several times
+  // over, fewer rows (more workgroups) for small batches.
+  const int64_t wgs8 = a.num_tokens * (a.h_out / 8);
+  int rs = wgs8 >= 2048 ? 8 : (wgs8 >= 512 ? 4 : 2);
+  if (tuning().bgmv_shrink_rows > 0) rs = tuning().bgmv_shrink_rows;
+  switch (rs) {
+    case 8:
+      return launch_shrink_rs<D, 8>(a, stream);
+    case 4:
+      return launch_shrink_rs<D, 4>(a, stream);
+    default:
+      return launch_shrink_rs<D, 2>(a, stream);
+  }
+}
+
+template <typename D, int CP>
+static hipError_t launch_expand_cp(const BgmvArgs& a, hipStream_t stream) {
+  constexpr int U = 4;
+  constexpr int cols_per_wg = (kBgmvThreads / CP) * U;
+  dim3 grid((a.h_out + cols_per_wg - 1) / cols_per_wg, static_cast<unsigned>(a.num_tokens));
+  hipLaunchKernelGGL((bgmv_expand_kernel<D, CP, U>), grid, dim3(kBgmvThreads), 0, stream,
+                     static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x),
+                     a.w_ptrs, a.indices, static_cast<int>(a.num_tokens), a.h_in, a.h_out,
+                     a.y_offset, a.y_stride, a.layer_idx, a.scale);
+  return hipGetLastError();
+}
+
+template <typename D>
+static hipError_t launch_expand(const BgmvArgs& a, hipStream_t stream) {
+  const int chunks = a.h_in / 8;
+  if (chunks <= 1) return launch_expand_cp<D, 1>(a, stream);
+  if (chunks <= 2) return launch_expand_cp<D, 2>(a, stream);
+  if (chunks <= 4) return launch_expand_cp<D, 4>(a, stream);
+  if (chunks <= 8) return launch_expand_cp<D, 8>(a, stream);
+  return launch_expand_cp<D, 16>(a, stream);
+}
+
+hipError_t launch_bgmv(const BgmvArgs& a, hipStream_t stream) {
+  const bool expand = a.h_in < a.h_out;  // bgmv_impl.cuh:204
+  if (a.dtype == LORAX_F16)
+    return expand ? launch_expand<F16>(a, stream) : launch_shrink<F16>(a, stream);
+  return expand ? launch_expand<BF16>(a, stream) : launch_shrink<BF16>(a, stream);
+}
+
+}  // namespace lorax

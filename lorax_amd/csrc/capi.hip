@@ -1,0 +1,241 @@
+// C ABI of liblorax_hip.so: argument validation, error reporting, per-device
+// workspace and dispatch to the kernel launchers.  The checks mirror the TORCH_CHECKs
+// of the reference's pybind layer (punica_kernels/punica_ops.cc:291-411); what that
+// layer reads from tensor metadata arrives here as plain integers.
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+
+#include "kernels.h"
+
+namespace lorax {
+namespace {
+
+constexpr int kMaxDevices = 64;
+constexpr int kMaxRank = 128;  // BGMV_MAX_RANK / MAX_RANK_CUSTOM, punica.py:37-39
+
+struct Workspace {
+  float* partials = nullptr;
+  uint32_t* counters = nullptr;
+};
+Workspace g_ws[kMaxDevices];
+std::mutex g_ws_mutex;
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int env_int(const char* name) {
+  const char* s = getenv(name);
+  return s ? atoi(s) : 0;
+}
+
+int init_device(int device) {
+  if (device < 0 || device >= kMaxDevices) return fail(LORAX_EINVAL, "device %d out of range", device);
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  if (g_ws[device].partials != nullptr) return LORAX_OK;
+  int prev = 0;
+  hipError_t e = hipGetDevice(&prev);
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (prev != device) {
+    e = hipSetDevice(device);
+    if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
+  }
+  float* partials = nullptr;
+  uint32_t* counters = nullptr;
+  e = hipMalloc(reinterpret_cast<void**>(&partials), kPartialBytes);
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&counters), kNumCounters * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipMemset(counters, 0, kNumCounters * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  if (prev != device) (void)hipSetDevice(prev);
+  if (e != hipSuccess) {
+    if (partials) (void)hipFree(partials);
+    if (counters) (void)hipFree(counters);
+    return fail(LORAX_ELAUNCH, "workspace allocation on device %d: %s", device, hipGetErrorString(e));
+  }
+  g_ws[device].partials = partials;
+  g_ws[device].counters = counters;
+  return LORAX_OK;
+}
+
+// Workspace of the current device; allocates it on first use unless `stream` is
+// being captured (allocation is not a capturable operation).
+Workspace current_workspace(hipStream_t stream) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return Workspace{};
+  if (g_ws[device].partials == nullptr) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) == hipSuccess && status == hipStreamCaptureStatusNone)
+      (void)init_device(device);
+  }
+  return g_ws[device];
+}
+
+int check_common(const void* y, const void* x, const void* w_ptrs, int dtype) {
+  if (y == nullptr || x == nullptr || w_ptrs == nullptr)
+    return fail(LORAX_EINVAL, "null pointer argument (y=%p x=%p w_ptrs=%p)", y, x, w_ptrs);
+  if (!aligned16(y) || !aligned16(x))
+    return fail(LORAX_EINVAL, "y and x must be 16-byte aligned (y=%p x=%p)", y, x);
+  if (dtype != LORAX_F16 && dtype != LORAX_BF16)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d (only f16=0 and bf16=1)", dtype);
+  return LORAX_OK;
+}
+
+}  // namespace
+
+const Tuning& tuning() {
+  static const Tuning t = {env_int("LORAX_BGMV_SHRINK_ROWS"), env_int("LORAX_SHRINK_KSPLIT"),
+                           env_int("LORAX_SHRINK_MB")};
+  return t;
+}
+
+}  // namespace lorax
+
+using namespace lorax;
+
+extern "C" {
+
+int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* indices,
+               int64_t num_tokens, int32_t h_in, int32_t h_out, int64_t y_offset,
+               int64_t y_stride, int64_t layer_idx, float scale, int32_t dtype, void* stream) {
+  if (num_tokens < 0) return fail(LORAX_EINVAL, "num_tokens=%lld is negative", (long long)num_tokens);
+  if (num_tokens == 0) return LORAX_OK;
+  if (int rc = check_common(y, x, w_ptrs, dtype)) return rc;
+  if (indices == nullptr) return fail(LORAX_EINVAL, "null pointer argument (indices)");
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  const bool expand = h_in < h_out;
+  const int narrow = expand ? h_in : h_out;
+  const int wide = expand ? h_out : h_in;
+  // punica_ops.cc:310 (dims < 65536) and bgmv_config.h:12-86 (narrow side 8..128).
+  if (h_in <= 0 || h_out <= 0 || h_in >= 65536 || h_out >= 65536 || narrow % 8 != 0 ||
+      narrow > kMaxRank || wide % 8 != 0)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. h_in=%d h_out=%d dtype=%d", h_in, h_out, dtype);
+  if (num_tokens > 65535)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. num_tokens=%lld exceeds 65535",
+                (long long)num_tokens);
+  if (y_offset < 0 || y_stride < y_offset + h_out)
+    return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld do not hold h_out=%d columns",
+                (long long)y_offset, (long long)y_stride, h_out);
+  BgmvArgs a{y, x, w_ptrs, indices, num_tokens, h_in, h_out, y_offset, y_stride, layer_idx, scale, dtype};
+  const hipError_t e = launch_bgmv(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
+int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
+                      const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
+                      int32_t h_in, int32_t r, int32_t a_layout, int64_t layer_idx, void* tmp,
+                      int64_t tmp_bytes, int32_t dtype, void* stream) {
+  if (num_segments < 0 || num_tokens < 0)
+    return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments,
+                (long long)num_tokens);
+  // Same contract as the reference: the custom kernel wants the 8 MiB buffer
+  // (punica_ops.cc:389-390), the cutlass path 60 bytes per problem (punica_ops.cc:359).
+  if (a_layout == LORAX_A_RH) {
+    if (tmp_bytes != LORAX_SHRINK_TMP_BYTES)
+      return fail(LORAX_ETMPSIZE, "CHECK_EQ(tmp.size(0), 8 * 1024 * 1024) failed. %lld vs %d",
+                  (long long)tmp_bytes, LORAX_SHRINK_TMP_BYTES);
+  } else if (a_layout == LORAX_A_HR) {
+    if (tmp_bytes != static_cast<int64_t>(lorax_sgmv_tmp_size(num_segments)))
+      return fail(LORAX_ETMPSIZE, "CHECK_EQ(tmp.size(0), sgmv_tmp_size(num_problems)) failed. %lld vs %zu",
+                  (long long)tmp_bytes, lorax_sgmv_tmp_size(num_segments));
+  } else {
+    return fail(LORAX_EINVAL, "a_layout=%d (0 = [L,r,h_in], 1 = [L,h_in,r])", a_layout);
+  }
+  if (num_segments == 0 || num_tokens == 0) return LORAX_OK;
+  if (int rc = check_common(v, x, w_ptrs, dtype)) return rc;
+  if (s_start == nullptr || s_end == nullptr || (tmp == nullptr && tmp_bytes > 0))
+    return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p tmp=%p)", s_start, s_end, tmp);
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  const bool r_ok = a_layout == LORAX_A_RH ? (r >= 16 && r <= kMaxRank && r % 16 == 0)
+                                           : (r >= 8 && r <= kMaxRank && r % 8 == 0);
+  if (!r_ok || h_in <= 0 || h_in % 8 != 0 || num_tokens > INT32_MAX / 2)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in,
+                r, a_layout);
+  const hipStream_t st = static_cast<hipStream_t>(stream);
+  const Workspace ws = current_workspace(st);
+  SgmvArgs a{};
+  a.y = v;
+  a.x = x;
+  a.w_ptrs = w_ptrs;
+  a.s_start = s_start;
+  a.s_end = s_end;
+  a.num_segments = num_segments;
+  a.num_tokens = num_tokens;
+  a.d_in = h_in;
+  a.d_out = r;
+  a.a_layout = a_layout;
+  a.layer_idx = layer_idx;
+  a.dtype = dtype;
+  a.partials = ws.partials;
+  a.partial_bytes = ws.partials ? kPartialBytes : 0;
+  a.counters = ws.counters;
+  a.num_counters = ws.counters ? kNumCounters : 0;
+  const hipError_t e = launch_sgmv_shrink(a, st);
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_shrink launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
+int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
+                      const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
+                      int32_t h_out, int64_t y_offset, int64_t y_stride, int64_t layer_idx,
+                      void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
+  if (num_segments < 0 || num_tokens < 0)
+    return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments,
+                (long long)num_tokens);
+  if (tmp_bytes != static_cast<int64_t>(lorax_sgmv_tmp_size(num_segments)))  // punica_ops.cc:359
+    return fail(LORAX_ETMPSIZE, "CHECK_EQ(tmp.size(0), sgmv_tmp_size(num_problems)) failed. %lld vs %zu",
+                (long long)tmp_bytes, lorax_sgmv_tmp_size(num_segments));
+  if (num_segments == 0 || num_tokens == 0) return LORAX_OK;
+  if (int rc = check_common(y, v, w_ptrs, dtype)) return rc;
+  if (s_start == nullptr || s_end == nullptr || (tmp == nullptr && tmp_bytes > 0))
+    return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p tmp=%p)", s_start, s_end, tmp);
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  if (r < 8 || r > kMaxRank || r % 8 != 0 || h_out <= 0 || h_out % 8 != 0 ||
+      num_tokens > INT32_MAX / 2)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d", dtype, r, h_out);
+  if (y_offset < 0 || y_offset % 8 != 0 || y_stride % 8 != 0 || y_stride < y_offset + h_out)
+    return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld must be multiples of 8 holding h_out=%d columns",
+                (long long)y_offset, (long long)y_stride, h_out);
+  SgmvArgs a{};
+  a.y = y;
+  a.x = v;
+  a.w_ptrs = w_ptrs;
+  a.s_start = s_start;
+  a.s_end = s_end;
+  a.num_segments = num_segments;
+  a.num_tokens = num_tokens;
+  a.d_in = r;
+  a.d_out = h_out;
+  a.y_offset = y_offset;
+  a.y_stride = y_stride;
+  a.layer_idx = layer_idx;
+  a.dtype = dtype;
+  const hipError_t e = launch_sgmv_expand(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_expand launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
+size_t lorax_sgmv_tmp_size(int32_t num_problems) {
+  // 3 pointers + 3 int64 leading dimensions + one (m, n, k) int32 triple per problem
+  return num_problems > 0 ? static_cast<size_t>(num_problems) * (3 * 8 + 3 * 8 + 12) : 0;
+}
+
+int lorax_init(int32_t device) { return init_device(device); }
+
+size_t lorax_workspace_bytes(void) { return kPartialBytes + kNumCounters * sizeof(uint32_t); }
+
+const char* lorax_last_error(void) { return g_error; }
+
+const char* lorax_version(void) { return "lorax_hip 0.1.0 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,175 @@
+// Shared device helpers for the gfx950 LoRA kernels: 16-bit float element traits,
+// 128-bit vector access, wave64 reductions and the token-grouping scan used by BGMV.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lorax {
+
+constexpr int kWave = 64;
+
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+// Element traits.  E is the 16-bit storage type; vec8 is eight of them (16 bytes).
+struct F16 {
+  using E = _Float16;
+  using vec8 = f16x8;
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+struct BF16 {
+  using E = __bf16;
+  using vec8 = bf16x8;
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename D>
+__device__ __forceinline__ float to_f32(typename D::E v) {
+  return static_cast<float>(v);
+}
+// Round-to-nearest-even conversion to the storage type.
+template <typename D>
+__device__ __forceinline__ typename D::E from_f32(float v) {
+  return static_cast<typename D::E>(v);
+}
+
+// y <- D(float(y) + float(D(delta))): the reference's two rounding points
+// (bgmv_impl.cuh:141, layers.py:190,210).
+template <typename D>
+__device__ __forceinline__ typename D::E accumulate(typename D::E y, float delta) {
+  return from_f32<D>(to_f32<D>(y) + to_f32<D>(from_f32<D>(delta)));
+}
+
+// Four adjacent elements (8 bytes, 8-byte aligned) updated with one load and one store.
+template <typename D>
+__device__ __forceinline__ void accumulate4(typename D::E* p, f32x4 delta) {
+  typedef typename D::E vec4 __attribute__((ext_vector_type(4)));
+  vec4 y = *reinterpret_cast<const vec4*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) y[i] = accumulate<D>(y[i], delta[i]);
+  *reinterpret_cast<vec4*>(p) = y;
+}
+
+template <typename D>
+__device__ __forceinline__ typename D::vec8 load8(const typename D::E* p) {
+  return *reinterpret_cast<const typename D::vec8*>(p);
+}
+template <typename D>
+__device__ __forceinline__ void store8(typename D::E* p, typename D::vec8 v) {
+  *reinterpret_cast<typename D::vec8*>(p) = v;
+}
+template <typename D>
+__device__ __forceinline__ typename D::vec8 zero8() {
+  typename D::vec8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = static_cast<typename D::E>(0.0f);
+  return z;
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+// Sum over the 64 lanes of a wave; every lane receives the total.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+}
+
+// Reduces N per-lane values across the wave with N-1+log2(64/N) shuffles instead of
+// 6*N: at every step a lane hands half of its values to the partner lane and keeps
+// the sum of the other half.  On return lane l holds in vals[0] the wave-wide total
+// of the input value with index transpose_reduce_index<N>(l).
+template <int N>
+__device__ __forceinline__ void transpose_reduce(float (&vals)[N]) {
+  static_assert(N >= 1 && N <= 64 && (N & (N - 1)) == 0, "N must be a power of two <= 64");
+  const int lane = lane_id();
+  int n = N;
+  int m = 32;
+#pragma unroll
+  for (; n > 1; n >>= 1, m >>= 1) {
+    const bool upper = (lane & m) != 0;
+    const int half = n >> 1;
+#pragma unroll
+    for (int i = 0; i < N / 2; ++i) {
+      if (i < half) {
+        const float keep = upper ? vals[i + half] : vals[i];
+        const float send = upper ? vals[i] : vals[i + half];
+        vals[i] = keep + __shfl_xor(send, m, kWave);
+      }
+    }
+  }
+#pragma unroll
+  for (; m >= 1; m >>= 1) vals[0] += __shfl_xor(vals[0], m, kWave);
+}
+
+// Index of the input value whose total lane `lane` holds after transpose_reduce<N>.
+template <int N>
+__device__ __forceinline__ int transpose_reduce_index(int lane) {
+  int idx = 0;
+  int n = N;
+  int m = 32;
+  for (; n > 1; n >>= 1, m >>= 1) {
+    if (lane & m) idx += n >> 1;
+  }
+  return idx;
+}
+
+// Token grouping for BGMV.  Tokens that share indices[] value share one adapter; the
+// tokens of one adapter are cut, in token order, into chunks of at most G and the
+// first token of each chunk ("leader") processes the whole chunk, so the adapter's
+// weights are fetched once per chunk instead of once per token.
+//
+// Called by every wave of the workgroup of token b with identical arguments; all
+// results are wave-uniform.  Returns the number of tokens in b's chunk (>= 1) if b
+// leads a chunk, with toks[0] = b and toks[1..] the followers in ascending order;
+// returns 0 if b is a follower (the workgroup has nothing to do).
+template <int G>
+__device__ __forceinline__ int group_tokens(const int64_t* __restrict__ indices, int num_tokens,
+                                            int b, int64_t idx, int (&toks)[G]) {
+  const int lane = lane_id();
+  toks[0] = b;
+#pragma unroll
+  for (int g = 1; g < G; ++g) toks[g] = b;
+  if (G == 1) return 1;
+
+  // Rank of b among the tokens of its adapter = matches strictly before b.
+  int before = 0;
+  const int b_blk = b & ~(kWave - 1);
+  for (int t0 = 0; t0 < b_blk; t0 += kWave) {
+    const bool same = indices[t0 + lane] == idx;  // t0 + lane < b_blk <= num_tokens
+    before += __popcll(__ballot(same));
+  }
+  int n = 1;
+  for (int t0 = b_blk; t0 < num_tokens; t0 += kWave) {
+    const int t = t0 + lane;
+    const bool same = (t < num_tokens) && (indices[t] == idx);
+    uint64_t mask = __ballot(same);
+    if (t0 == b_blk) {
+      const uint64_t below = (1ull << (b - b_blk)) - 1ull;
+      before += __popcll(mask & below);
+      if ((before % G) != 0) return 0;
+      mask &= ~(below | (1ull << (b - b_blk)));
+    }
+    while (mask != 0 && n < G) {
+      const int pos = __ffsll(static_cast<unsigned long long>(mask)) - 1;
+      mask &= mask - 1;
+#pragma unroll
+      for (int g = 1; g < G; ++g) {
+        if (g == n) toks[g] = t0 + pos;
+      }
+      ++n;
+    }
+    if (n == G) break;
+  }
+  return n;
+}
+
+}  // namespace lorax

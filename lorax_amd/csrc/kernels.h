@@ -1,0 +1,66 @@
+// Internal interface between the C ABI (capi.hip) and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/lorax_hip.h"
+#include "common.h"
+
+namespace lorax {
+
+struct BgmvArgs {
+  void* y;
+  const void* x;
+  const int64_t* w_ptrs;
+  const int64_t* indices;
+  int64_t num_tokens;
+  int h_in;
+  int h_out;
+  int64_t y_offset;
+  int64_t y_stride;
+  int64_t layer_idx;
+  float scale;
+  int dtype;
+};
+
+struct SgmvArgs {
+  void* y;        // v for shrink, y for expand
+  const void* x;  // x for shrink, v for expand
+  const int64_t* w_ptrs;
+  const int32_t* s_start;
+  const int32_t* s_end;
+  int num_segments;
+  int64_t num_tokens;
+  int d_in;
+  int d_out;
+  int a_layout;  // shrink only
+  int64_t y_offset;
+  int64_t y_stride;
+  int64_t layer_idx;
+  int dtype;
+  // library workspace of the current device (shrink split-K)
+  float* partials;
+  size_t partial_bytes;
+  uint32_t* counters;
+  size_t num_counters;
+};
+
+// Launch parameters that can be overridden from the environment for tuning runs
+// (LORAX_BGMV_SHRINK_ROWS, LORAX_SHRINK_KSPLIT, LORAX_SHRINK_MB); 0 = heuristic.
+struct Tuning {
+  int bgmv_shrink_rows;
+  int shrink_ksplit;
+  int shrink_mb;
+};
+const Tuning& tuning();
+
+hipError_t launch_bgmv(const BgmvArgs& a, hipStream_t stream);
+hipError_t launch_sgmv_shrink(const SgmvArgs& a, hipStream_t stream);
+hipError_t launch_sgmv_expand(const SgmvArgs& a, hipStream_t stream);
+
+// Workspace layout constants shared by capi.hip and sgmv_shrink.hip.
+constexpr size_t kPartialBytes = 96u << 20;  // fp32 split-K partial sums
+constexpr size_t kNumCounters = 1u << 18;    // one arrival counter per row tile
+
+}  // namespace lorax

@@ -1,0 +1,223 @@
+// SGMV expand for gfx950: y[s:e, off:off+h_out] += T(v[s:e, :r] @ B_i), B_i = [r, h_out].
+//
+// Replaces the expand configuration of the reference's cutlass grouped GEMM
+// (sgmv/sgmv_cutlass.cuh:86-131; problem set-up :30-52).
+//
+// The contraction is only r (<= 128) long and the output is huge, so the kernel is a
+// read-modify-write stream over y.  A workgroup owns 64 output columns of one row
+// chunk of one segment:
+//   * long segments: the r x 64 panel of B goes through LDS once, every wave turns it
+//     into MFMA operands that stay in registers, and then walks 16-row blocks of the
+//     chunk computing the transposed product (B^T as the first MFMA operand, v as the
+//     second), which leaves each lane with 8 adjacent columns of one y row per pair of
+//     accumulators - y is read and written with 16-byte accesses and never staged;
+//   * segments of a few rows (decode tokens inside a prefill batch): MFMA operand
+//     set-up would dominate, so the panel is streamed row by row on the vector ALU
+//     with 16-byte loads, each lane owning 8 adjacent columns.
+#include "kernels.h"
+#include "sgmv_tiles.h"
+
+namespace lorax {
+
+constexpr int kExpandWaves = 4;
+constexpr int kExpandThreads = kExpandWaves * kWave;
+constexpr int kExpandCols = 64;          // output columns per workgroup
+constexpr int kExpandBlocksPerWave = 4;  // 16-row blocks per wave and tile
+constexpr int kExpandRows = 16 * kExpandWaves * kExpandBlocksPerWave;  // rows per tile
+constexpr int kExpandShortRows = 4;      // row tiles up to this height use the vector path
+constexpr int kPanelPitch = kExpandCols + 4;  // LDS row pitch in elements
+
+// Output column (0..63) that row `a` of the first MFMA operand of accumulator j
+// stands for.  Chosen so that lane group g = a / 4 ends up with columns
+// [8g, 8g+8) in accumulators 0,1 and [32+8g, 32+8g+8) in accumulators 2,3.
+__device__ __forceinline__ int panel_col(int j, int a) {
+  return (j >> 1) * 32 + (a >> 2) * 8 + (j & 1) * 4 + (a & 3);
+}
+
+template <typename D, int KS>
+__global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
+    typename D::E* __restrict__ Y, const typename D::E* __restrict__ V,
+    const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
+    const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int r, int h_out,
+    int64_t y_offset, int64_t y_stride, int64_t layer_idx) {
+  using E = typename D::E;
+  using vec8 = typename D::vec8;
+  __shared__ __attribute__((aligned(16))) E panel[KS * 32 * kPanelPitch];
+  __shared__ float redf[kExpandWaves][kExpandCols];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int c = lane & 15;
+  const int g = lane >> 4;
+  const int n0 = blockIdx.x * kExpandCols;
+
+  for (int tile = blockIdx.y;; tile += gridDim.y) {
+    RowTile rt;
+    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, kExpandRows, tile, rt)) break;
+    const E* B = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * r * static_cast<int64_t>(h_out);
+    const int nrows = rt.row_end - rt.row0;
+    if (nrows <= kExpandShortRows) {
+      // ---- vector path: thread (kq, c8) owns k = kq, kq+32, ... and 8 columns ----
+      const int c8 = tid & 7;
+      const int kq = tid >> 3;
+      const int col = n0 + c8 * 8;
+      float bw[KS][8];
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int k = kq + 32 * s;
+        vec8 bv = zero8<D>();
+        if (k < r && col < h_out) bv = load8<D>(B + static_cast<int64_t>(k) * h_out + col);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bw[s][e] = to_f32<D>(bv[e]);
+      }
+      for (int row = rt.row0; row < rt.row_end; ++row) {
+        float part[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part[e] = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          const int k = kq + 32 * s;
+          const float vk = k < r ? to_f32<D>(V[static_cast<int64_t>(row) * r + k]) : 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) part[e] = fmaf(vk, bw[s][e], part[e]);
+        }
+        // lanes of a wave are (kq % 8, c8): fold the eight kq of the wave together
+#pragma unroll
+        for (int m = 8; m < kWave; m <<= 1)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) part[e] += __shfl_xor(part[e], m, kWave);
+        if (lane < 8) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) redf[wave][c8 * 8 + e] = part[e];
+        }
+        __syncthreads();
+        if (tid < kExpandCols && n0 + tid < h_out) {
+          float s = 0.f;
+#pragma unroll
+          for (int w = 0; w < kExpandWaves; ++w) s += redf[w][tid];
+          E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0 + tid;
+          *yp = accumulate<D>(*yp, s);
+        }
+        __syncthreads();
+      }
+      continue;
+    }
+
+    // ---- MFMA path ----
+    // Stage the r x 64 panel of B in LDS (rows k >= r and columns >= h_out as zeros).
+    for (int p = tid; p < KS * 32 * (kExpandCols / 8); p += kExpandThreads) {
+      const int k = p / (kExpandCols / 8);
+      const int cc = (p % (kExpandCols / 8)) * 8;
+      vec8 bv = zero8<D>();
+      if (k < r && n0 + cc < h_out) bv = load8<D>(B + static_cast<int64_t>(k) * h_out + n0 + cc);
+      // rows are 8-byte aligned (pitch 68 elements), so two 8-byte LDS stores
+      const u32x4 bits = __builtin_bit_cast(u32x4, bv);
+      u32x2* dst = reinterpret_cast<u32x2*>(panel + k * kPanelPitch + cc);
+      dst[0] = u32x2{bits[0], bits[1]};
+      dst[1] = u32x2{bits[2], bits[3]};
+    }
+    __syncthreads();
+    vec8 bf[4][KS];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int colj = panel_col(j, c);
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bf[j][s][e] = panel[(s * 32 + g * 8 + e) * kPanelPitch + colj];
+    }
+    __syncthreads();  // the panel may be overwritten by the next tile from here on
+
+    const int nmb = (nrows + 15) / 16;
+    const bool col_ok0 = n0 + g * 8 < h_out;
+    const bool col_ok1 = n0 + 32 + g * 8 < h_out;
+    auto load_block = [&](int mb, vec8(&vf)[KS], vec8& y0, vec8& y1) {
+      const int row = rt.row0 + mb * 16 + c;
+      const bool ok = row < rt.row_end;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        vf[s] = zero8<D>();
+        if (ok && s * 32 + g * 8 < r) vf[s] = load8<D>(V + static_cast<int64_t>(row) * r + s * 32 + g * 8);
+      }
+      const E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0 + g * 8;
+      y0 = zero8<D>();
+      y1 = zero8<D>();
+      if (ok && col_ok0) y0 = load8<D>(yp);
+      if (ok && col_ok1) y1 = load8<D>(yp + 32);
+    };
+    auto finish_block = [&](int mb, const vec8(&vf)[KS], vec8 y0, vec8 y1) {
+      f32x4 acc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s) acc[j] = D::mfma16(bf[j][s], vf[s], acc[j]);
+      }
+      const int row = rt.row0 + mb * 16 + c;
+      const bool ok = row < rt.row_end;
+      E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0 + g * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        y0[i] = accumulate<D>(y0[i], acc[0][i]);
+        y0[4 + i] = accumulate<D>(y0[4 + i], acc[1][i]);
+        y1[i] = accumulate<D>(y1[i], acc[2][i]);
+        y1[4 + i] = accumulate<D>(y1[4 + i], acc[3][i]);
+      }
+      if (ok && col_ok0) store8<D>(yp, y0);
+      if (ok && col_ok1) store8<D>(yp + 32, y1);
+    };
+
+    int mb = wave;
+    if (mb < nmb) {
+      vec8 va[KS], vb[KS], ya0, ya1, yb0, yb1;
+      load_block(mb, va, ya0, ya1);
+      while (true) {
+        const int mb2 = mb + kExpandWaves;
+        if (mb2 < nmb) load_block(mb2, vb, yb0, yb1);
+        finish_block(mb, va, ya0, ya1);
+        if (mb2 >= nmb) break;
+        const int mb3 = mb2 + kExpandWaves;
+        if (mb3 < nmb) load_block(mb3, va, ya0, ya1);
+        finish_block(mb2, vb, yb0, yb1);
+        if (mb3 >= nmb) break;
+        mb = mb3;
+      }
+    }
+  }
+}
+
+template <typename D, int KS>
+static hipError_t launch_expand_ks(const SgmvArgs& a, hipStream_t stream) {
+  const int64_t tiles = (a.num_tokens + kExpandRows - 1) / kExpandRows + a.num_segments;
+  dim3 grid((a.d_out + kExpandCols - 1) / kExpandCols,
+            static_cast<unsigned>(tiles < 65535 ? tiles : 65535));
+  hipLaunchKernelGGL((sgmv_expand_kernel<D, KS>), grid, dim3(kExpandThreads), 0, stream,
+                     static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x),
+                     a.w_ptrs, a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens),
+                     a.d_in, a.d_out, a.y_offset, a.y_stride, a.layer_idx);
+  return hipGetLastError();
+}
+
+template <typename D>
+static hipError_t launch_expand_dtype(const SgmvArgs& a, hipStream_t stream) {
+  switch ((a.d_in + 31) / 32) {
+    case 1:
+      return launch_expand_ks<D, 1>(a, stream);
+    case 2:
+      return launch_expand_ks<D, 2>(a, stream);
+    case 3:
+      return launch_expand_ks<D, 3>(a, stream);
+    case 4:
+      return launch_expand_ks<D, 4>(a, stream);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_sgmv_expand(const SgmvArgs& a, hipStream_t stream) {
+  return a.dtype == LORAX_F16 ? launch_expand_dtype<F16>(a, stream)
+                              : launch_expand_dtype<BF16>(a, stream);
+}
+
+}  // namespace lorax

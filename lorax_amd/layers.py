@@ -1,0 +1,178 @@
+"""LoRA-augmented linear layers: the callers of the SGMV/BGMV kernels.
+
+Mirrors ``lorax_server/utils/layers.py:59-300``: ``LoraLinear.forward_layer_type`` (the
+"legacy punica" branch, :107-167), ``TensorParallelMultiAdapterLinear`` (fused q/k/v and
+gate/up outputs, one column slice per layer name, :217-255) and
+``TensorParallelAdapterRowLinear`` (o_proj / down_proj, :270-289).
+
+Two deliberate differences from the reference:
+  * its third branch, the per-adapter masked matmul loop (:169-211), is not part of this
+    package: a batch the kernels cannot take raises instead of silently running dense
+    PyTorch code;
+  * a projection that owns only a column slice of the fused output is written in place
+    through the kernels' column window instead of through a zero-filled staging tensor
+    and a second pass (:109-112,166-167).  Every token belongs to at most one rank
+    group, so both orders round identically.
+"""
+
+from typing import List, Optional
+
+import torch
+from torch import nn
+
+from lorax_amd.adapters import LORA, AdapterBatchData, BatchLoraWeights
+from lorax_amd.sgmv import (
+    add_lora_a_bgmv,
+    add_lora_b_bgmv,
+    add_lora_b_bgmv_slice,
+    has_sgmv,
+    lora_a_sgmv_cutlass,
+    lora_b_sgmv_cutlass,
+    lora_b_sgmv_cutlass_slice,
+)
+
+
+class SingleProcessGroup:
+    """A process group of one rank (the reference's FakeGroup, utils/dist.py:19-45)."""
+
+    def size(self) -> int:
+        return 1
+
+    def rank(self) -> int:
+        return 0
+
+
+class LoraLinear(nn.Module):
+    def __init__(self, base_layer, layer_id: int, process_group=None):
+        super().__init__()
+        self.base_layer = base_layer
+        self.layer_id = layer_id
+        self.process_group = process_group if process_group is not None else SingleProcessGroup()
+
+    def forward_layer_type(
+        self,
+        result: torch.Tensor,
+        input: torch.Tensor,
+        adapter_data: AdapterBatchData,
+        layer_type: str,
+        start_idx: int,
+        end_idx: int,
+    ) -> torch.Tensor:
+        layer_data = adapter_data.data.get(layer_type)
+        data: Optional[BatchLoraWeights] = layer_data.get(LORA) if layer_data is not None else None
+        if data is None:
+            return result  # no adapter in the batch targets this projection
+        if not has_sgmv():
+            raise RuntimeError("LoRA kernels unavailable: liblorax_hip.so is not loaded or DISABLE_SGMV is set")
+        if not data.can_vectorize(self.process_group):
+            raise RuntimeError(
+                f"layer type {layer_type!r}: ranks {sorted(data.rank_data)} are outside what the LoRA kernels "
+                "cover (rank / world_size <= 128, not lm_head)"
+            )
+
+        sliced = end_idx - start_idx != result.shape[1]
+        tensor_parallel = self.process_group.size() > 1
+        for r, rank_segments in data.rank_data.items():
+            a_ptr, b_ptr = rank_segments.lora_a_ptr, rank_segments.lora_b_ptr
+            if a_ptr is None or b_ptr is None:
+                continue
+            if data.use_sgmv:
+                v = lora_a_sgmv_cutlass(
+                    input,
+                    rank_segments.tmp_shrink,
+                    a_ptr,
+                    rank_segments.segment_starts,
+                    rank_segments.segment_ends,
+                    self.layer_id,
+                    r,
+                )
+                if tensor_parallel:
+                    v = self.collect_lora_a(v)
+                if sliced:
+                    lora_b_sgmv_cutlass_slice(
+                        result,
+                        v,
+                        rank_segments.tmp_expand,
+                        b_ptr,
+                        rank_segments.segment_starts,
+                        rank_segments.segment_ends,
+                        self.layer_id,
+                        start_idx,
+                        end_idx - start_idx,
+                    )
+                else:
+                    lora_b_sgmv_cutlass(
+                        result,
+                        v,
+                        rank_segments.tmp_expand,
+                        b_ptr,
+                        rank_segments.segment_starts,
+                        rank_segments.segment_ends,
+                        self.layer_id,
+                    )
+            else:
+                v = torch.zeros((input.size(0), r), dtype=input.dtype, device=input.device)
+                add_lora_a_bgmv(v, input, a_ptr, rank_segments.indices, self.layer_id)
+                if tensor_parallel:
+                    v = self.collect_lora_a(v)
+                if sliced:
+                    add_lora_b_bgmv_slice(
+                        result, v, b_ptr, rank_segments.indices, self.layer_id, start_idx, end_idx - start_idx
+                    )
+                else:
+                    add_lora_b_bgmv(result, v, b_ptr, rank_segments.indices, self.layer_id)
+        return result
+
+    def collect_lora_a(self, a_out: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError("tensor-parallel exchange of the shrink output is outside this package")
+
+
+class TensorParallelMultiAdapterLinear(LoraLinear):
+    """Column-parallel projection(s) sharing one input: q/k/v or gate/up (utils/layers.py:217-255)."""
+
+    def __init__(self, base_layer, layer_id: int, layer_names: List[str], sizes: Optional[List[int]], process_group=None):
+        super().__init__(base_layer, layer_id, process_group)
+        self.layer_names = layer_names
+        self.sizes = sizes
+
+    @classmethod
+    def load(cls, base_layer, layer_id, layer_names, sizes, process_group=None):
+        return cls(base_layer, layer_id, layer_names, sizes, process_group)
+
+    def forward(self, input: torch.Tensor, adapter_data: AdapterBatchData) -> torch.Tensor:
+        result = self.base_layer(input)
+        out_shape = result.shape
+        if input.dim() >= 3:
+            # (batch, seq, hidden) models: the kernels want one row per token
+            input = input.reshape(-1, input.shape[-1])
+            result = result.reshape(-1, result.shape[-1])
+        world = self.process_group.size()
+        offset = 0
+        for i, name in enumerate(self.layer_names):
+            start = offset // world
+            if self.sizes is not None:
+                offset += self.sizes[i]
+                end = offset // world
+            else:
+                end = result.shape[1]
+            result = self.forward_layer_type(result, input, adapter_data, name, start, end)
+        return result.reshape(out_shape)
+
+
+class TensorParallelAdapterRowLinear(LoraLinear):
+    """Row-parallel projection: o_proj / down_proj (utils/layers.py:270-289)."""
+
+    def __init__(self, base_layer, layer_id: int, layer_name: str, process_group=None):
+        super().__init__(base_layer, layer_id, process_group)
+        self.layer_name = layer_name
+
+    @classmethod
+    def load(cls, base_layer, layer_id, layer_name, process_group=None):
+        return cls(base_layer, layer_id, layer_name, process_group)
+
+    def forward(self, input: torch.Tensor, adapter_data: AdapterBatchData) -> torch.Tensor:
+        result = self.base_layer(input)
+        stride = result.shape[-1] // self.process_group.size()
+        start = self.process_group.rank() * stride
+        self.forward_layer_type(result, input, adapter_data, self.layer_name, start, start + stride)
+        return result

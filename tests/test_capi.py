@@ -1,0 +1,92 @@
+"""The C-ABI shared library without a GPU: it loads, exports every function include/lorax_hip.h
+declares, and rejects bad arguments on the host before anything is launched."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from lorax_amd import _native
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = (ROOT / "include" / "lorax_hip.h").read_text()
+
+
+def _declared_functions():
+    body = re.sub(r"/\*.*?\*/", "", HEADER, flags=re.S)
+    return sorted(set(re.findall(r"\b(lorax_[a-z0-9_]+)\s*\(", body)))
+
+
+def test_library_loads():
+    assert _native.available(), _native.load_error()
+    assert "gfx950" in _native.version()
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    declared = _declared_functions()
+    assert "lorax_bgmv" in declared and "lorax_sgmv_shrink" in declared and "lorax_sgmv_expand" in declared
+    raw = ctypes.CDLL(str(_native.LIB_PATH))
+    for name in declared:
+        assert hasattr(raw, name), f"{name} is declared in lorax_hip.h but not exported"
+    assert sorted(_native.EXPORTED_SYMBOLS) == declared
+
+
+def test_tmp_size_is_60_bytes_per_problem():
+    lib = _native.lib()
+    assert [lib.lorax_sgmv_tmp_size(n) for n in (-1, 0, 1, 32, 257)] == [0, 0, 60, 1920, 15420]
+    assert lib.lorax_workspace_bytes() > 8 * 1024 * 1024
+
+
+OK, EINVAL, ENOKERNEL, ELAUNCH, ETMPSIZE = 0, 1, 2, 3, 4
+P = 0x1000  # a non-null, 16-byte aligned fake address: validation failures return before any launch
+
+
+def _err():
+    return _native.lib().lorax_last_error().decode()
+
+
+def test_bgmv_validation():
+    f = _native.lib().lorax_bgmv
+    assert f(None, None, None, None, 0, 4096, 8, 0, 8, 0, 1.0, 1, None) == OK  # nothing to do
+    assert f(None, P, P, P, 4, 4096, 8, 0, 8, 0, 1.0, 1, None) == EINVAL and "null" in _err()
+    assert f(P, P + 2, P, P, 4, 4096, 8, 0, 8, 0, 1.0, 1, None) == EINVAL and "aligned" in _err()
+    assert f(P, P, P, P, 4, 4096, 8, 0, 8, 0, 1.0, 2, None) == ENOKERNEL and "No suitable kernel" in _err()
+    for h_in, h_out in [(4096, 12), (4096, 136), (4100, 8), (65536, 8), (8, 65536), (256, 256)]:
+        assert f(P, P, P, P, 4, h_in, h_out, 0, h_out, 0, 1.0, 1, None) == ENOKERNEL, (h_in, h_out)
+        assert f"h_in={h_in} h_out={h_out}" in _err()
+    assert f(P, P, P, P, 4, 8, 4096, 8192, 8192, 0, 1.0, 1, None) == EINVAL  # window outside the row
+    assert f(P, P, P, P, -1, 8, 4096, 0, 4096, 0, 1.0, 1, None) == EINVAL
+    assert f(P, P, P, P, 4, 8, 4096, 0, 4096, -1, 1.0, 1, None) == EINVAL
+
+
+def test_sgmv_shrink_validation():
+    f = _native.lib().lorax_sgmv_shrink
+    big = 8 * 1024 * 1024
+    assert f(P, P, P, P, P, 2, 16, 4096, 16, 0, 0, P, big - 1, 0, None) == ETMPSIZE and "8 * 1024 * 1024" in _err()
+    assert f(P, P, P, P, P, 2, 16, 4096, 8, 1, 0, P, 119, 0, None) == ETMPSIZE and "sgmv_tmp_size" in _err()
+    assert f(P, P, P, P, P, 0, 16, 4096, 16, 0, 0, P, big, 0, None) == OK  # no segments
+    assert f(P, P, P, P, P, 2, 16, 4096, 16, 7, 0, P, big, 0, None) == EINVAL  # layout
+    for r in (8, 24, 144):
+        assert f(P, P, P, P, P, 2, 16, 4096, r, 0, 0, P, big, 0, None) == ENOKERNEL, r
+    assert f(P, P, P, P, P, 2, 16, 4100, 16, 0, 0, P, big, 0, None) == ENOKERNEL
+    assert f(P, P, P, None, P, 2, 16, 4096, 16, 0, 0, P, big, 0, None) == EINVAL
+    assert f(P, P, P, P, P, 2, 16, 4096, 16, 0, 0, P, big, 5, None) == ENOKERNEL  # dtype
+
+
+def test_sgmv_expand_validation():
+    f = _native.lib().lorax_sgmv_expand
+    assert f(P, P, P, P, P, 2, 16, 16, 4096, 0, 4096, 0, P, 121, 1, None) == ETMPSIZE
+    assert f(P, P, P, P, P, 0, 16, 16, 4096, 0, 4096, 0, None, 0, 1, None) == OK
+    for r, h in [(4, 4096), (136, 4096), (16, 4100)]:
+        assert f(P, P, P, P, P, 2, 16, r, h, 0, h, 0, P, 120, 1, None) == ENOKERNEL, (r, h)
+    assert f(P, P, P, P, P, 2, 16, 16, 4096, 4, 8192, 0, P, 120, 1, None) == EINVAL  # unaligned window
+    assert f(P, P, P, P, P, 2, 16, 16, 4096, 4096, 4096, 0, P, 120, 1, None) == EINVAL  # window too wide
+
+
+def test_python_binding_rejects_cpu_tensors():
+    import torch
+
+    y = torch.zeros(2, 8, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        _native.dispatch_bgmv(y, y, torch.zeros(1, dtype=torch.int64), torch.zeros(2, dtype=torch.int64), 0, 1.0)

@@ -1,0 +1,243 @@
+"""Host-side mirror of the reference API (no GPU): routing tables, padding, orientation, the
+scratch-size contract - against the reference tests' golden vectors and against the oracle."""
+
+import json
+from pathlib import Path
+from unittest import mock
+
+import pytest
+import torch
+
+from lorax_amd import punica, sgmv
+from lorax_amd.adapters import (
+    LORA,
+    LM_HEAD,
+    AdapterBatchData,
+    AdapterBatchMetadata,
+    AdapterWeights,
+    BatchAdapterWeights,
+    LayerAdapterWeights,
+    LoraConfig,
+    LoraWeights,
+    get_scaling_factor,
+)
+from lorax_amd.segments import SegmentConcatBuilder, find_segments
+from oracle import lora_oracle as O
+
+GOLDEN = Path(__file__).resolve().parent / "golden"
+
+
+def _golden(name):
+    return json.loads((GOLDEN / f"{name}.json").read_text())
+
+
+def test_surface_matches_reference_names():
+    for name in ["MIN_SGMV_RANK", "MIN_RANK_CUSTOM", "MAX_RANK_CUSTOM", "SGMV_BLOCK_SIZE", "BGMV_MAX_RANK",
+                 "LORAX_PUNICA_TRITON_DISABLED", "has_sgmv", "pad_rank", "pad_to_min_rank", "use_cutlass_shrink",
+                 "orient_for_rank", "add_lora_sgmv_cutlass", "lora_a_sgmv_cutlass", "lora_b_sgmv_cutlass",
+                 "add_lora_a_bgmv", "add_lora_b_bgmv", "get_tmp_tensor", "get_tmp_tensors",
+                 "get_tmp_tensor_for_size", "get_tmp_expand_size", "segmented_matmul"]:
+        assert hasattr(sgmv, name), name
+        assert getattr(punica, name) is getattr(sgmv, name), name
+    assert (sgmv.MIN_SGMV_RANK, sgmv.MIN_RANK_CUSTOM, sgmv.MAX_RANK_CUSTOM, sgmv.SGMV_BLOCK_SIZE,
+            sgmv.BGMV_MAX_RANK) == (8, 16, 128, 16, 128)
+
+
+@pytest.mark.parametrize("case", _golden("segments")["find_segments"])
+@pytest.mark.parametrize("as_tensor", [True, False])
+def test_find_segments_golden(case, as_tensor):
+    arg = torch.tensor(case["adapter_indices"]) if as_tensor else case["adapter_indices"]
+    assert find_segments(arg) == (case["segments"], case["segment_indices"])
+
+
+def test_find_segments_matches_oracle_on_random_runs():
+    g = torch.Generator().manual_seed(5)
+    for n in [1, 2, 7, 64, 513]:
+        idx = torch.randint(-1, 4, (n,), generator=g)
+        assert find_segments(idx) == O.find_segments_ref(idx.tolist())
+
+
+@pytest.mark.parametrize("case", _golden("segments")["concat_segments"])
+def test_concat_segments_golden(case):
+    builder = SegmentConcatBuilder()
+    for seg, idx in case["batches"]:
+        builder.concat(torch.tensor(seg), idx)
+    segments, owners = builder.build()
+    assert segments.tolist() == case["segments"]
+    assert owners == case["segment_indices"]
+    assert O.concat_segments_ref(case["batches"]) == (case["segments"], case["segment_indices"])
+
+
+@pytest.mark.parametrize("world_size", _golden("sgmv_kat")["pad_rank"]["world_sizes"])
+@pytest.mark.parametrize("lora_rank", _golden("sgmv_kat")["pad_rank"]["lora_ranks"])
+def test_pad_rank(lora_rank, world_size):
+    assert sgmv.has_sgmv(), "the shared library must load on a machine without a GPU too"
+    kat = _golden("sgmv_kat")["pad_rank"]
+    x = torch.randn((kat["bs"], kat["h"]), dtype=torch.float16)
+    a = torch.randn((kat["h"], lora_rank), dtype=torch.float16)
+    b = torch.randn((lora_rank, kat["h"]), dtype=torch.float16)
+    ap = sgmv.pad_rank(a, dim=1, world_size=world_size)
+    bp = sgmv.pad_rank(b, dim=0, world_size=world_size)
+    assert ap.size(1) == bp.size(0) >= lora_rank
+    assert torch.equal(ap, O.pad_to_min_rank_ref(a, 1, 8 * world_size))
+    assert torch.equal(bp, O.pad_to_min_rank_ref(b, 0, 8 * world_size))
+    assert torch.allclose(x @ a @ b, x @ ap @ bp)
+
+
+def test_orient_and_cutlass_shrink_rules():
+    t = torch.zeros(6, 4)
+    for r in [1, 8, 15, 16, 64, 128, 129, 256]:
+        assert sgmv.use_cutlass_shrink(r) == (r < 16)
+        assert sgmv.orient_for_rank(t, r).shape == O.orient_for_rank_ref(t, r).shape
+    assert sgmv.orient_for_rank(t, 16).data_ptr() == t.data_ptr()  # a view, not a copy
+
+
+def test_scaling_factor():
+    assert get_scaling_factor(16, 8) == 2.0
+    assert get_scaling_factor(16, 64, uses_rslora=True) == 2.0
+
+
+def test_tmp_size_contract():
+    for n in [0, 1, 2, 32, 257]:
+        assert sgmv.get_tmp_expand_size(n) == O.sgmv_tmp_size_ref(n)
+
+
+def _meta(adapter_indices, segments=None, segment_indices=None, adapter_list=None):
+    if segments is None:
+        segments, segment_indices = find_segments(adapter_indices)
+    return AdapterBatchMetadata(
+        adapter_indices=torch.tensor(adapter_indices, dtype=torch.int64),
+        adapter_list=adapter_list if adapter_list is not None else adapter_indices,
+        adapter_set=set(adapter_indices),
+        adapter_segments=torch.tensor(segments, dtype=torch.int64),
+        segment_indices=segment_indices,
+    )
+
+
+def _layer(ranks, h=1024):
+    layer = LayerAdapterWeights()
+    assert layer.is_empty()
+    for idx, r in enumerate(ranks):
+        w = LoraWeights([torch.randn((h, r), dtype=torch.float16)], [torch.randn((r, h), dtype=torch.float16)],
+                        LoraConfig(r=r))
+        assert w.lora_a_r == r and w.lora_b_r == r
+        layer.add_adapter(idx, w)
+    assert not layer.is_empty()
+    return layer
+
+
+@pytest.mark.parametrize("lora_ranks", _golden("lora_batch")["prefill"]["rank_sets"])
+def test_batched_lora_weights_prefill(lora_ranks):
+    gp = _golden("lora_batch")["prefill"]
+    h = gp["h"]
+    layer = _layer(lora_ranks, h)
+    meta = _meta(gp["adapter_indices"], gp["adapter_segments"], gp["segment_indices"], gp["adapter_list"])
+    with mock.patch("lorax_amd.adapters.get_tmp_tensors", return_value=(torch.empty(0), torch.empty(0))):
+        data = layer.get_data(meta, LM_HEAD, prefill=True, prefill_head_indices=None).get(LORA)
+    assert data.use_sgmv
+    assert data.lora_a.keys() == meta.adapter_set and data.lora_b.keys() == meta.adapter_set
+    for i, r in enumerate(lora_ranks):
+        assert data.lora_a[i].shape == ((1, h, r) if r < gp["min_rank_custom"] else (1, r, h))
+        assert data.lora_b[i].shape == (1, r, h)
+    assert data.rank_data.keys() == set(lora_ranks)
+    n = gp["entries_per_rank_group"]
+    for r, rd in data.rank_data.items():
+        assert rd.rank == r
+        assert rd.lora_a_ptr.shape == rd.lora_b_ptr.shape == rd.segment_starts.shape == rd.segment_ends.shape == (n,)
+        assert rd.indices is None
+    # rank group of adapter 0 owns runs 0 and 2
+    rd0 = data.rank_data[lora_ranks[0]]
+    assert rd0.segment_starts.tolist() == [0, 4] and rd0.segment_ends.tolist() == [2, 6]
+    assert rd0.lora_a_ptr.tolist() == [layer.adapter_weights[0].weights_a.data_ptr()] * 2
+    assert rd0.lora_b_ptr.tolist() == [layer.adapter_weights[0].weights_b.data_ptr()] * 2
+
+
+@pytest.mark.parametrize("case", _golden("lora_batch")["decode"])
+def test_batched_lora_weights_decode(case):
+    layer = _layer(case["lora_ranks"])
+    meta = _meta(case["adapter_indices"])
+    data = layer.get_data(meta, LM_HEAD, prefill=False, prefill_head_indices=None).get(LORA)
+    assert not data.use_sgmv
+    assert {str(r) for r in data.rank_data} == set(case["expected"])
+    oracle = O.rank_groups_ref(meta.segment_indices, case["adapter_indices"],
+                               {i: r for i, r in enumerate(case["lora_ranks"])})
+    for r, rd in data.rank_data.items():
+        exp = case["expected"][str(r)]
+        assert rd.lora_a_ptr.shape == rd.lora_b_ptr.shape == (exp["num_ptrs"],)
+        assert rd.indices.dtype == torch.int64 and rd.indices.tolist() == exp["indices"] == oracle[r][1]
+        assert rd.segment_starts is None and rd.segment_ends is None
+        assert rd.tmp_shrink is None and rd.tmp_expand is None
+        # decode pointers address the [L, r, h_in] / [L, h_out, r] stacks of the run owners
+        owners = [meta.segment_indices[p] for p in oracle[r][0]]
+        assert rd.lora_a_ptr.tolist() == [layer.adapter_weights[a].weights_a_t.data_ptr() for a in owners]
+        assert rd.lora_b_ptr.tolist() == [layer.adapter_weights[a].weights_b_t.data_ptr() for a in owners]
+
+
+class _OtherWeights(AdapterWeights):
+    @classmethod
+    def get_batch_types(cls):
+        return [_OtherBatch]
+
+
+class _OtherBatch(BatchAdapterWeights):
+    def has_adapter(self, adapter_index):
+        return False
+
+    @classmethod
+    def key(cls):
+        return "other"
+
+    @classmethod
+    def load(cls, adapter_weights, meta, layer_name, prefill, prefill_head_indices):
+        return None
+
+
+def test_batch_with_no_lora_segment_yields_nothing():
+    g = _golden("lora_batch")["no_lora_segments"]
+    layer = LayerAdapterWeights()
+    layer.add_adapter(0, _OtherWeights())
+    r = g["lora_rank"]
+    layer.add_adapter(g["lora_adapter"], LoraWeights([torch.randn(64, r)], [torch.randn(r, 64)], LoraConfig(r=r)))
+    meta = _meta(g["adapter_indices"], g["adapter_segments"], g["segment_indices"], g["adapter_list"])
+    assert layer.get_data(meta, LM_HEAD, prefill=True, prefill_head_indices=None) == {}
+    batch = AdapterBatchData.from_meta(meta, {"q_proj": layer}, {}, None, True, None)
+    assert batch.data == {} and batch.max_rank == 0 and batch.ranks() == set()
+
+
+def test_lora_weights_layouts_stay_resident():
+    h_in, h_out = 64, 48
+    for r in [8, 16]:
+        a = [torch.randn(h_in, r) for _ in range(3)]
+        b = [torch.randn(r, h_out) for _ in range(3)]
+        w = LoraWeights(a, b, LoraConfig(r=r))
+        assert w.weights_a.shape == ((3, h_in, r) if r < 16 else (3, r, h_in))
+        assert w.weights_b.shape == (3, r, h_out)
+        assert w.weights_a_t.shape == (3, r, h_in) and w.weights_b_t.shape == (3, h_out, r)
+        ptrs = (w.weights_a.data_ptr(), w.weights_b.data_ptr(), w.weights_a_t.data_ptr(), w.weights_b_t.data_ptr())
+        for _ in range(2):  # alternating prefill / decode accesses never move a stack
+            assert ptrs == (w.weights_a.data_ptr(), w.weights_b.data_ptr(), w.weights_a_t.data_ptr(),
+                            w.weights_b_t.data_ptr())
+        assert torch.equal(w.weights_a_t[1], a[1].t()) and torch.equal(w.weights_b_t[2], b[2].t())
+
+
+def test_from_peft_folds_scale_and_pads():
+    r, h_in, h_out = 4, 32, 24
+    A = [torch.randn(r, h_in)]
+    B = [torch.randn(h_out, r)]
+    cfg = LoraConfig(r=r, lora_alpha=8)
+    w = LoraWeights.from_peft(A, B, cfg)
+    assert cfg.r == 8 and w.lora_a_r == 8
+    x = torch.randn(5, h_in)
+    expect = (x @ A[0].t() @ B[0].t()) * 2.0
+    assert torch.allclose(x @ w.weights_a[0] @ w.weights_b[0], expect, atol=1e-5)
+
+
+def test_segmented_matmul():
+    x = torch.randn(6, 8)
+    w = [torch.randn(4, 8), torch.randn(4, 8), torch.randn(4, 8)]
+    b = [torch.randn(4), None, torch.randn(4)]
+    y = torch.zeros(6, 4)
+    sgmv.segmented_matmul(y, x, w, b, torch.tensor([0, 3, 2], dtype=torch.int32), torch.tensor([2, 6, 2], dtype=torch.int32))
+    assert torch.allclose(y[0:2], x[0:2] @ w[0].t() + b[0])
+    assert torch.allclose(y[3:6], x[3:6] @ w[1].t())
+    assert torch.count_nonzero(y[2]) == 0
