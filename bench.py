@@ -1,0 +1,336 @@
+"""Benchmark of the multi-adapter LoRA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {1,2,3,4,5}] [--layers L]
+
+A step is one pass of one synthetic batch through the LoRA computation of `layers` decoder
+layers (every projection of the configuration: zero-fill of v, shrink, expand), issued through
+the reference-shaped API and replayed as one HIP graph, with all inputs resident in HBM.
+The default configuration is the BGMV decode batch: 256 bf16 tokens over 128 resident rank-8
+adapters, 5 % of the tokens without adapter, LoRA on q/k/v/o (4096/1024/1024/4096).
+
+Prints ONE JSON line: metric/value = tokens x layers per second of the whole step; "roofline" =
+algorithmic HBM bytes per launch of the kernel that takes most of the step divided by its average
+launch duration, measured with events on the launch stream around graphs holding only that
+kernel; "cpu_baseline" = the oracle's restatement of the reference's per-adapter masked matmul
+loop timed on the host cores on one layer of the same batch.
+"""
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
+    p.add_argument("--layers", type=int, default=0, help="layers per step (0 = the configuration's default)")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--eager", action="store_true", help="launch every step eagerly instead of replaying a graph")
+    return p.parse_args()
+
+
+def build_workload(cfg: int, layers: int, device):
+    from lorax_amd import synthetic
+
+    defaults = {1: 32, 2: 32, 3: 8, 4: 2, 5: 1}
+    L = layers or defaults[cfg]
+    if cfg == 5:
+        return synthetic.config5(device, num_layers=L, weights_on_device=True)
+    return synthetic.CONFIGS[cfg](device, num_layers=L, weights_on_device=True)
+
+
+class Plan:
+    """Pre-built kernel arguments of one workload: per projection the rank groups' tables plus the
+    static v and y buffers, and closures that issue the zero-fill / shrink / expand launches."""
+
+    def __init__(self, w):
+        import torch
+
+        from lorax_amd.adapters import LORA
+
+        self.w = w
+        self.batch = w.batch_data()
+        self.calls = []  # (kind, fn, algorithmic bytes, flops) in issue order for ONE layer; fn(layer)
+        e = 2
+        T = w.num_tokens
+        for group in w.groups:
+            x = w.inputs[group.name]
+            y = torch.zeros((T, group.h_out), dtype=w.dtype, device=w.device)
+            off = 0
+            for name, size in zip(group.layer_names, group.sizes):
+                data = self.batch.data.get(name, {}).get(LORA)
+                if data is not None:
+                    for r, rd in data.rank_data.items():
+                        self._add_rank_group(data.use_sgmv, x, y, off, size, group, r, rd, e)
+                off += size
+
+    def _add_rank_group(self, use_sgmv, x, y, off, size, group, r, rd, e):
+        import torch
+
+        from lorax_amd import sgmv
+
+        T = x.size(0)
+        v = torch.zeros((T, r), dtype=x.dtype, device=x.device)
+        if use_sgmv:
+            lens = (rd.segment_ends - rd.segment_starts).clamp(min=0)
+            rows = int(lens.sum().item())
+            uniq = len(set(rd.lora_a_ptr[lens > 0].tolist()))
+            starts, ends, tmp_s, tmp_e = rd.segment_starts, rd.segment_ends, rd.tmp_shrink, rd.tmp_expand
+            a_ptr, b_ptr = rd.lora_a_ptr, rd.lora_b_ptr
+            a_is_rh = not sgmv.use_cutlass_shrink(r)
+
+            def shrink(layer):
+                if a_is_rh:
+                    sgmv._kernels.sgmv_shrink(v, x, a_ptr, starts, ends, tmp_s, layer)
+                else:
+                    sgmv._kernels.sgmv_cutlass(v, x, a_ptr, starts, ends, tmp_s, layer)
+
+            def expand(layer):
+                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_ptr, starts, ends, layer, off, size)
+
+            kind = "sgmv"
+        else:
+            routed = rd.indices >= 0
+            rows = int(routed.sum().item())
+            uniq = len(set(rd.lora_a_ptr[rd.indices[routed]].tolist()))
+            idx, a_ptr, b_ptr = rd.indices, rd.lora_a_ptr, rd.lora_b_ptr
+
+            def shrink(layer):
+                sgmv.add_lora_a_bgmv(v, x, a_ptr, idx, layer)
+
+            def expand(layer):
+                sgmv.add_lora_b_bgmv_slice(y, v, b_ptr, idx, layer, off, size)
+
+            kind = "bgmv"
+        h_in = group.h_in
+        shrink_bytes = rows * h_in * e + uniq * r * h_in * e + rows * r * e
+        expand_bytes = rows * r * e + uniq * r * size * e + 2 * rows * size * e
+        self.calls.append(("zero", lambda layer: v.zero_(), 0, 0))
+        self.calls.append((f"{kind}_shrink", shrink, shrink_bytes, 2 * rows * r * h_in))
+        self.calls.append((f"{kind}_expand", expand, expand_bytes, 2 * rows * r * size))
+
+    def issue(self, layers, kinds=None):
+        n = 0
+        for layer in range(layers):
+            for kind, fn, _, _ in self.calls:
+                if kinds is None or kind in kinds:
+                    fn(layer)
+                    n += 1
+        return n
+
+    def bytes_per_layer(self, kind=None):
+        return sum(b for k, _, b, _ in self.calls if kind is None or k == kind)
+
+    def launches_per_layer(self, kind):
+        return sum(1 for k, _, _, _ in self.calls if k == kind)
+
+
+def capture(plan, layers, kinds=None):
+    import torch
+
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        plan.issue(1, kinds)  # warm up lazily-initialised state outside the capture
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        n = plan.issue(layers, kinds)
+    return graph, n
+
+
+def time_graph(graph, reps, warmup=3):
+    """Average duration of one replay in ms, from events recorded on the stream the replays run on."""
+    import torch
+
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        graph.replay()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / reps
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """The reference's per-adapter masked matmul loop (oracle) on the host cores: one layer of the same
+    batch, every projection; the adapter set is cut to a prefix if the full loop would blow the budget
+    and the time is scaled linearly (the loop is linear in the number of adapters)."""
+    import torch
+
+    from oracle import lora_oracle as O
+
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    idx = torch.tensor(w.adapter_indices)
+    active = sorted({a for a in w.adapter_indices if a in w.rank_of_adapter})
+    xs = {g.name: w.inputs[g.name].cpu() for g in w.groups}
+
+    def run(adapters):
+        t0 = time.perf_counter()
+        for g in w.groups:
+            result = torch.zeros((w.num_tokens, g.h_out), dtype=w.dtype)
+            off = 0
+            for name, size in zip(g.layer_names, g.sizes):
+                layer = w.weights[name].adapter_weights
+                la = {a: layer[a].weights_a[:1].cpu() for a in adapters if a in layer}
+                lb = {a: layer[a].weights_b[:1].cpu() for a in adapters if a in layer}
+                t1 = time.perf_counter()
+                O.fallback_layer_type(result, xs[g.name], idx, adapters, la, lb, 0, off, off + size)
+                run.compute += time.perf_counter() - t1
+                off += size
+        return time.perf_counter() - t0
+
+    run.compute = 0.0
+    probe = active[: max(1, min(len(active), 4))]
+    run(probe)  # warm-up, also sizes the sample
+    run.compute = 0.0
+    run(probe)
+    per_adapter = run.compute / len(probe)
+    n = max(1, min(len(active), int(budget_s / 3 / max(per_adapter, 1e-9))))
+    sample = active[:n]
+    times = []
+    for _ in range(3 if n == len(active) else 1):
+        run.compute = 0.0
+        run(sample)
+        times.append(run.compute)
+    t_layer = statistics.median(times) * (len(active) / n)
+    note = f"{n} of {len(active)} active adapters, 1 layer, all projections"
+    if n < len(active):
+        note += " (time extrapolated linearly in the adapter count)"
+    return {
+        "value": w.num_tokens / t_layer,
+        "unit": "tokens/s per LoRA layer",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": note,
+        "seconds_per_layer": t_layer,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; --gpus above 1 is not supported by this build", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from lorax_amd import _native
+
+    if not _native.available():
+        raise RuntimeError(f"liblorax_hip.so is missing: {_native.load_error()}")
+    if not torch.cuda.is_available():
+        raise RuntimeError("bench.py needs a GPU")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    _native.init(device)
+
+    w = build_workload(args.config, args.layers, device)
+    L = w.num_layers
+    plan = Plan(w)
+    torch.cuda.synchronize()
+
+    if args.eager:
+        run_step = lambda: plan.issue(L)  # noqa: E731
+    else:
+        graph, launches = capture(plan, L)
+        run_step = graph.replay
+
+    for _ in range(args.warmup):
+        run_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    tokens_per_s = w.num_tokens * L / (elapsed / args.steps)
+
+    # per-kernel timing: graphs that hold only one kind of launch, over the same layer sweep
+    kinds = sorted({k for k, _, _, _ in plan.calls if k != "zero"})
+    per_kind = {}
+    for kind in kinds:
+        g, n = capture(plan, L, kinds={kind})
+        ms = time_graph(g, reps=max(5, min(50, args.steps)))
+        avg_us = ms * 1e3 / n
+        bytes_per_launch = plan.bytes_per_layer(kind) / plan.launches_per_layer(kind)
+        per_kind[kind] = {
+            "launches_per_layer": plan.launches_per_layer(kind),
+            "avg_launch_us": avg_us,
+            "bytes_per_launch": bytes_per_launch,
+            "GBps": bytes_per_launch / (avg_us * 1e-6) / 1e9,
+            "share_ms": ms,
+        }
+        del g
+    dominant = max(per_kind, key=lambda k: per_kind[k]["share_ms"])
+    dk = per_kind[dominant]
+    traffic = None
+    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(traffic_file):
+        traffic = json.load(open(traffic_file)).get(f"cfg{args.config}", {}).get(dominant)
+
+    out = {
+        "metric": "LoRA-layer tokens/sec (BGMV decode / SGMV prefill), HBM roofline fraction in 'roofline'",
+        "value": tokens_per_s,
+        "unit": "tokens/s per LoRA layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": w.name,
+            "tokens": w.num_tokens,
+            "routed_tokens": w.routed_tokens(),
+            "distinct_adapters": w.distinct_adapters(),
+            "resident_adapters": len(w.rank_of_adapter),
+            "layers_per_step": L,
+            "projections": [n for g in w.groups for n in g.layer_names],
+            "launch": "eager" if args.eager else "hip_graph",
+            "algorithmic_bytes_per_layer": plan.bytes_per_layer(),
+            "step_GBps": plan.bytes_per_layer() * L / (elapsed / args.steps) / 1e9,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": dominant,
+            "achieved": dk["GBps"],
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": dk["GBps"] / HBM_PEAK_GBS,
+            "traffic": traffic,
+            "avg_launch_us": dk["avg_launch_us"],
+            "bytes_per_launch": dk["bytes_per_launch"],
+        },
+        "kernels": per_kind,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

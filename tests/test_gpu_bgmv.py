@@ -1,0 +1,192 @@
+"""BGMV parity on the GPU: the HIP kernels, called through the C ABI by the reference-shaped
+wrappers (add_lora_a_bgmv / add_lora_b_bgmv), against the CPU oracle on the same seeded inputs.
+Tolerance: max-abs <= 2e-2 and relative L2 <= 5e-3; routing (which rows change) is bit-exact."""
+
+import pytest
+import torch
+
+from lorax_amd import _native, sgmv
+from oracle import lora_oracle as O
+from tests.helpers import assert_close, ptr_table, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _stacks(n, L, rows, cols, gen, dtype, std=0.02):
+    return [randn((L, rows, cols), std, gen, dtype, DEV) for _ in range(n)]
+
+
+def _indices(T, n_adapters, gen, drop=0.1):
+    idx = torch.randint(0, n_adapters, (T,), generator=gen)
+    idx[torch.rand((T,), generator=gen) < drop] = -1
+    return idx
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("r", [8, 16, 32, 64, 128])
+@pytest.mark.parametrize("T,h_in,h_out,n_adapters", [(1, 1024, 1024, 1), (7, 4096, 1024, 3), (256, 4096, 4096, 24),
+                                                     (33, 14336, 4096, 12)])
+def test_bgmv_shrink_expand_vs_oracle(dtype, r, T, h_in, h_out, n_adapters):
+    print(f"case dtype={dtype} r={r} T={T} h_in={h_in} h_out={h_out}", flush=True)
+    gen = torch.Generator().manual_seed(100 + r + T)
+    L, layer = 3, 2
+    wa_t = _stacks(n_adapters, L, r, h_in, gen, dtype)   # [L, r, h_in]
+    wb_t = _stacks(n_adapters, L, h_out, r, gen, dtype)  # [L, h_out, r]
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    y0 = randn((T, h_out), 0.5, gen, dtype, DEV)
+    idx = _indices(T, n_adapters, gen)
+    idx_d = idx.to(DEV)
+    # entries no token refers to hold a null pointer and must never be dereferenced
+    unused = [a for a in range(n_adapters) if a not in set(idx.tolist())]
+    wa_ptr = ptr_table(wa_t, DEV, null_at=unused)
+    wb_ptr = ptr_table(wb_t, DEV, null_at=unused)
+
+    v = torch.zeros((T, r), dtype=dtype, device=DEV)
+    sgmv.add_lora_a_bgmv(v, x, wa_ptr, idx_d, layer)
+    y = y0.clone()
+    sgmv.add_lora_b_bgmv(y, v, wb_ptr, idx_d, layer)
+    torch.cuda.synchronize()
+
+    v_ref = torch.zeros((T, r), dtype=dtype)
+    O.bgmv_ref(v_ref, x.cpu(), [w.cpu() for w in wa_t], idx.tolist(), layer)
+    y_ref = y0.cpu().clone()
+    O.bgmv_ref(y_ref, v_ref, [w.cpu() for w in wb_t], idx.tolist(), layer)
+
+    assert_close(v, v_ref, "shrink output v")
+    assert_close(y, y_ref, "expand output y")
+    assert_close(y.float() - y0.float(), y_ref.float() - y0.cpu().float(), "delta")
+    untouched = idx < 0
+    assert torch.equal(y.cpu()[untouched], y0.cpu()[untouched])
+    assert torch.count_nonzero(v.cpu()[untouched]) == 0
+
+
+@pytest.mark.parametrize("r", [24, 48, 96, 120])
+def test_bgmv_ranks_that_are_not_powers_of_two(r):
+    print(f"case r={r}", flush=True)
+    gen = torch.Generator().manual_seed(r)
+    dtype, T, h_in, h_out, n, L = torch.bfloat16, 19, 2752, 1152, 5, 2
+    wa_t = _stacks(n, L, r, h_in, gen, dtype)
+    wb_t = _stacks(n, L, h_out, r, gen, dtype)
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    idx = _indices(T, n, gen)
+    v = torch.zeros((T, r), dtype=dtype, device=DEV)
+    y = torch.zeros((T, h_out), dtype=dtype, device=DEV)
+    sgmv.add_lora_a_bgmv(v, x, ptr_table(wa_t, DEV), idx.to(DEV), 1)
+    sgmv.add_lora_b_bgmv(y, v, ptr_table(wb_t, DEV), idx.to(DEV), 1)
+    v_ref = torch.zeros((T, r), dtype=dtype)
+    y_ref = torch.zeros((T, h_out), dtype=dtype)
+    O.bgmv_ref(v_ref, x.cpu(), [w.cpu() for w in wa_t], idx.tolist(), 1)
+    O.bgmv_ref(y_ref, v_ref, [w.cpu() for w in wb_t], idx.tolist(), 1)
+    assert_close(v, v_ref, "v")
+    assert_close(y, y_ref, "y")
+
+
+def test_bgmv_routing_is_bit_exact():
+    """Weights crafted so that the result names the adapter: A_i picks x[:, 0] (= 1), B_i column j is
+    (i + 1) / 256 + j / 16 in exactly representable values. Any routing slip changes bits."""
+    dtype, T, h_in, h_out, r, n, L, layer = torch.float16, 300, 256, 64, 8, 37, 2, 1
+    gen = torch.Generator().manual_seed(7)
+    idx = _indices(T, n, gen, drop=0.2)
+    wa_t, wb_t = [], []
+    for i in range(n):
+        a = torch.zeros(L, r, h_in)
+        a[layer, 0, 0] = 1.0
+        b = torch.zeros(L, h_out, r)
+        b[layer, :, 0] = (i + 1) / 256.0 + torch.arange(h_out) / 16.0
+        wa_t.append(a.to(dtype).to(DEV))
+        wb_t.append(b.to(dtype).to(DEV))
+    x = torch.zeros(T, h_in)
+    x[:, 0] = 1.0
+    x[:, 1:] = torch.randn(T, h_in - 1, generator=gen)
+    x = x.to(dtype).to(DEV)
+    v = torch.zeros((T, r), dtype=dtype, device=DEV)
+    y0 = torch.full((T, h_out), 0.25, dtype=dtype)
+    y = y0.to(DEV)
+    sgmv.add_lora_a_bgmv(v, x, ptr_table(wa_t, DEV), idx.to(DEV), layer)
+    sgmv.add_lora_b_bgmv(y, v, ptr_table(wb_t, DEV), idx.to(DEV), layer)
+    expect = y0.clone().float()
+    for t, i in enumerate(idx.tolist()):
+        if i >= 0:
+            expect[t] += (i + 1) / 256.0 + torch.arange(h_out) / 16.0
+    assert torch.equal(y.cpu(), expect.to(dtype))
+    exp_v = torch.zeros(T, r)
+    exp_v[idx >= 0, 0] = 1.0
+    assert torch.equal(v.cpu().float(), exp_v)
+
+
+def test_bgmv_column_window_of_fused_output():
+    dtype, T, h_in, r, n = torch.bfloat16, 40, 4096, 16, 6
+    sizes = [4096, 1024, 1024]
+    gen = torch.Generator().manual_seed(11)
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    idx = _indices(T, n, gen)
+    y0 = randn((T, sum(sizes)), 0.5, gen, dtype, DEV)
+    y = y0.clone()
+    y_ref = y0.cpu().clone()
+    off = 0
+    for h_out in sizes:
+        wa_t = _stacks(n, 1, r, h_in, gen, dtype)
+        wb_t = _stacks(n, 1, h_out, r, gen, dtype)
+        v = torch.zeros((T, r), dtype=dtype, device=DEV)
+        sgmv.add_lora_a_bgmv(v, x, ptr_table(wa_t, DEV), idx.to(DEV), 0)
+        sgmv.add_lora_b_bgmv_slice(y, v, ptr_table(wb_t, DEV), idx.to(DEV), 0, off, h_out)
+        v_ref = torch.zeros((T, r), dtype=dtype)
+        O.bgmv_ref(v_ref, x.cpu(), [w.cpu() for w in wa_t], idx.tolist(), 0)
+        part = y_ref[:, off:off + h_out].clone()
+        O.bgmv_ref(part, v_ref, [w.cpu() for w in wb_t], idx.tolist(), 0)
+        y_ref[:, off:off + h_out] = part
+        off += h_out
+    assert_close(y, y_ref, "fused q/k/v output")
+
+
+def test_bgmv_under_graph_capture_replays_identically():
+    dtype, T, h_in, h_out, r, n = torch.bfloat16, 64, 4096, 4096, 32, 9
+    gen = torch.Generator().manual_seed(3)
+    wa_t = _stacks(n, 2, r, h_in, gen, dtype)
+    wb_t = _stacks(n, 2, h_out, r, gen, dtype)
+    wa_ptr, wb_ptr = ptr_table(wa_t, DEV), ptr_table(wb_t, DEV)
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    idx = _indices(T, n, gen).to(DEV)
+    # graph padding rule of the reference (utils/graph.py:71-73,421-425): extra rows carry index -1
+    idx[-8:] = -1
+
+    def run(v, y):
+        v.zero_()
+        y.zero_()
+        sgmv.add_lora_a_bgmv(v, x, wa_ptr, idx, 1)
+        sgmv.add_lora_b_bgmv(y, v, wb_ptr, idx, 1)
+
+    v_e = torch.empty((T, r), dtype=dtype, device=DEV)
+    y_e = torch.empty((T, h_out), dtype=dtype, device=DEV)
+    run(v_e, y_e)
+    torch.cuda.synchronize()
+    v_g = torch.empty_like(v_e)
+    y_g = torch.empty_like(y_e)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(v_g, y_g)
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, y_e) and torch.equal(v_g, v_e)
+        y_g.fill_(7.0)  # eager work between replays
+
+
+def test_bgmv_errors_raise_runtime_error():
+    x = torch.zeros((4, 4096), dtype=torch.bfloat16, device=DEV)
+    ptr = torch.zeros(1, dtype=torch.int64, device=DEV)
+    idx = torch.full((4,), -1, dtype=torch.int64, device=DEV)
+    with pytest.raises(RuntimeError, match="No suitable kernel"):
+        sgmv.add_lora_a_bgmv(torch.zeros((4, 12), dtype=torch.bfloat16, device=DEV), x, ptr, idx, 0)
+    with pytest.raises(RuntimeError, match="No suitable kernel"):
+        sgmv.add_lora_a_bgmv(torch.zeros((4, 8), dtype=torch.float32, device=DEV), x.float(), ptr, idx, 0)
+    with pytest.raises(RuntimeError, match="CHECK_EQ"):
+        sgmv.add_lora_a_bgmv(torch.zeros((3, 8), dtype=torch.bfloat16, device=DEV), x, ptr, idx, 0)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        sgmv.add_lora_a_bgmv(torch.zeros((4, 16), dtype=torch.bfloat16, device=DEV)[:, ::2], x, ptr, idx, 0)
+    # all tokens at -1: a valid call that touches nothing
+    v = torch.ones((4, 8), dtype=torch.bfloat16, device=DEV)
+    sgmv.add_lora_a_bgmv(v, x, ptr, idx, 0)
+    assert torch.all(v == 1)
+    assert _native.available()

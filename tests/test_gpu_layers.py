@@ -1,0 +1,130 @@
+"""End-to-end parity of the LoRA layers on the five benchmark configurations: routing tables built by
+BatchLoraWeights, kernels called by LoraLinear.forward_layer_type, result compared with the
+reference's per-adapter masked matmul loop (the oracle's fallback_layer_type) on the same inputs.
+
+The oracle loop is dense over all tokens for every adapter, so it runs on reduced layer counts
+(the kernels index one layer of the stack; the others only occupy memory) and, for the largest
+shapes, on the LoRA delta of a subset of projections; full-size runs are checked through
+size-independent properties in test_gpu_properties.py."""
+
+import pytest
+import torch
+
+from lorax_amd import synthetic
+from lorax_amd.adapters import LORA
+from lorax_amd.layers import TensorParallelAdapterRowLinear, TensorParallelMultiAdapterLinear
+from oracle import lora_oracle as O
+from tests.helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+class ZeroBase(torch.nn.Module):
+    """Base projection that returns y0 (a fixed tensor) so the test isolates the LoRA path."""
+
+    def __init__(self, y0):
+        super().__init__()
+        self.y0 = y0
+
+    def forward(self, x):
+        return self.y0.clone()
+
+
+def _oracle_group(w, group, layer_id, y0_cpu):
+    x = w.inputs[group.name].cpu()
+    idx = torch.tensor(w.adapter_indices)
+    result = y0_cpu.clone()
+    off = 0
+    for name, size in zip(group.layer_names, group.sizes):
+        layer = w.weights[name]
+        lora_a = {a: lw.weights_a.cpu() for a, lw in layer.adapter_weights.items() if a in set(w.adapter_indices)}
+        lora_b = {a: lw.weights_b.cpu() for a, lw in layer.adapter_weights.items() if a in set(w.adapter_indices)}
+        O.fallback_layer_type(result, x, idx, set(w.adapter_indices), lora_a, lora_b, layer_id, off, off + size)
+        off += size
+    return result
+
+
+def _run_group(w, group, layer_id, y0, batch):
+    base = ZeroBase(y0)
+    x = w.inputs[group.name]
+    if len(group.layer_names) == 1 and group.name in ("o_proj", "down_proj"):
+        layer = TensorParallelAdapterRowLinear.load(base, layer_id, group.layer_names[0])
+    else:
+        sizes = group.sizes if len(group.layer_names) > 1 else None
+        layer = TensorParallelMultiAdapterLinear.load(base, layer_id, group.layer_names, sizes)
+    return layer(x, batch)
+
+
+def _check_workload(w, layer_id, y0_std):
+    batch = w.batch_data()
+    gen = torch.Generator().manual_seed(99)
+    untouched = torch.tensor([a not in w.rank_of_adapter for a in w.adapter_indices])
+    for group in w.groups:
+        print(f"{w.name}: group {group.name} T={w.num_tokens}", flush=True)
+        y0 = (torch.randn((w.num_tokens, group.h_out), generator=gen) * y0_std).to(w.dtype)
+        out = _run_group(w, group, layer_id, y0.to(DEV), batch)
+        torch.cuda.synchronize()
+        ref = _oracle_group(w, group, layer_id, y0)
+        assert_close(out, ref, f"{w.name}/{group.name}")
+        assert_close(out.float().cpu() - y0.float(), ref.float() - y0.float(), f"{w.name}/{group.name} delta")
+        assert torch.equal(out.cpu()[untouched], y0[untouched]), "rows without an adapter must be bit-identical"
+
+
+def test_config1_llama7b_q_proj_prefill():
+    w = synthetic.config1(DEV, num_layers=2)
+    assert w.meta.adapter_segments.tolist() == [0, 16, 32, 48, 64] and w.meta.segment_indices == [0, 1, 2, 3]
+    data = w.batch_data().data["q_proj"][LORA]
+    assert data.use_sgmv and list(data.rank_data) == [16]
+    _check_workload(w, 1, 0.5)
+    _check_workload(w, 0, 0.0)
+
+
+def test_config2_bgmv_decode_qkvo():
+    w = synthetic.config2(DEV, num_layers=2)
+    assert w.num_tokens == 256 and 0 < w.num_tokens - w.routed_tokens() < 40
+    data = w.batch_data().data["q_proj"][LORA]
+    assert not data.use_sgmv and list(data.rank_data) == [8]
+    _check_workload(w, 1, 0.25)
+    _check_workload(w, 0, 0.0)
+
+
+def test_config3_sgmv_prefill_mlp_reduced():
+    # same generator as the full configuration with shorter runs: 12 runs, lengths in [16, 300]
+    w = synthetic.config3(DEV, num_layers=2, num_segments=12, max_len=300)
+    assert all(rd.rank == 64 for rd in w.batch_data().data["gate_proj"][LORA].rank_data.values())
+    _check_workload(w, 1, 0.5)
+
+
+def test_config4_bgmv_multirank_decode_block():
+    w = synthetic.config4(DEV, num_layers=2, weights_on_device=False, num_tokens=512, resident_only_active=True)
+    batch = w.batch_data()
+    ranks = set(batch.data["q_proj"][LORA].rank_data)
+    assert ranks == {8, 16, 32, 64}
+    for rd in batch.data["down_proj"][LORA].rank_data.values():
+        members = (rd.indices >= 0).sum().item()
+        assert 0 < members < w.num_tokens  # every rank group leaves the others' tokens at -1
+    _check_workload(w, 1, 0.25)
+
+
+def test_config5_llama70b_mixed_batch_reduced():
+    # the real hidden sizes with a shorter prefill run and fewer decode tokens; attention projections
+    groups = [g for g in synthetic.LLAMA70B_LAYER if g.name in ("qkv", "o_proj")]
+    w = synthetic.config5(DEV, num_layers=1, weights_on_device=False, prefill_tokens=300, decode_tokens=24,
+                          num_adapters=16, groups=groups)
+    batch = w.batch_data()
+    data = batch.data["q_proj"][LORA]
+    assert data.use_sgmv and list(data.rank_data) == [128]
+    rd = data.rank_data[128]
+    lens = (rd.segment_ends - rd.segment_starts).tolist()
+    assert max(lens) >= 300 and lens.count(1) >= 10
+    # the run whose adapter has no weights and the run with no adapter are in no rank group
+    assert len(lens) < len(w.meta.segment_indices)
+    _check_workload(w, 0, 0.25)
+
+
+def test_config5_mlp_projections_reduced():
+    groups = [g for g in synthetic.LLAMA70B_LAYER if g.name in ("gate_up", "down_proj")]
+    w = synthetic.config5(DEV, num_layers=1, weights_on_device=False, prefill_tokens=130, decode_tokens=8,
+                          num_adapters=6, groups=groups)
+    _check_workload(w, 0, 0.25)

@@ -1,0 +1,251 @@
+"""SGMV parity on the GPU: shrink and expand HIP kernels through the C ABI (via the
+reference-shaped wrappers lora_a_sgmv_cutlass / lora_b_sgmv_cutlass) against the CPU oracle.
+Tolerance: max-abs <= 2e-2, relative L2 <= 5e-3; rows outside every segment stay bit-identical."""
+
+import json
+from pathlib import Path
+
+import pytest
+import torch
+
+from lorax_amd import sgmv
+from oracle import lora_oracle as O
+from tests.helpers import assert_close, ptr_table, randn, stored_sgmv_a
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+KAT = json.loads((Path(__file__).resolve().parent / "golden" / "sgmv_kat.json").read_text())
+
+
+def _run_pair(x, y, wa_list, wb_list, starts, ends, layer, r):
+    s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
+    wa_ptr = ptr_table(wa_list, DEV)
+    wb_ptr = ptr_table(wb_list, DEV)
+    tmp_shrink, tmp_expand = sgmv.get_tmp_tensors(len(starts), r, x.device)
+    v = sgmv.lora_a_sgmv_cutlass(x, tmp_shrink, wa_ptr, s_start, s_end, layer, r)
+    sgmv.lora_b_sgmv_cutlass(y, v, tmp_expand, wb_ptr, s_start, s_end, layer)
+    return v
+
+
+@pytest.mark.parametrize("segments", KAT["segments"])
+@pytest.mark.parametrize("lora_rank", KAT["lora_ranks"])
+def test_add_lora_sgmv_reference_kat(lora_rank, segments):
+    """The reference's own known-answer test (server/tests/utils/test_sgmv.py:42-105): same shapes,
+    seed, segment lists (the second has an empty segment behind a null pointer), tolerances and the
+    requirement that a graph-captured replay gives the same answer."""
+    print(f"case r={lora_rank} segments={segments}", flush=True)
+    torch.manual_seed(KAT["seed"])
+    B, H, r, L = KAT["B"], KAT["H"], lora_rank, KAT["nlayers"]
+    y = torch.zeros((B, H), dtype=torch.float16, device=DEV)
+    x = torch.randn((B, H), dtype=torch.float16, device=DEV)
+    wa = torch.randn(L, r, H, dtype=torch.float16, device=DEV)
+    if sgmv.use_cutlass_shrink(r):
+        wa = wa.transpose(1, 2).contiguous()
+    wb = torch.randn(L, r, H, dtype=torch.float16, device=DEV)
+    starts, ends = segments
+    wa_list = [wa if e - s > 0 else None for s, e in zip(starts, ends)]
+    wb_list = [wb if e - s > 0 else None for s, e in zip(starts, ends)]
+    layer = KAT["layer_idx"]
+
+    y_ref = O.sgmv_ref(y.clone(), x, wa_list, wb_list, starts, ends, layer, r)
+
+    y_ours = torch.zeros((B, H), dtype=torch.float16, device=DEV)
+    _run_pair(x, y_ours, wa_list, wb_list, starts, ends, layer, r)
+    assert torch.allclose(y_ref, y_ours, rtol=KAT["rtol"], atol=KAT["atol"]), (y_ref - y_ours).abs().max()
+
+    s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
+    wa_ptr, wb_ptr = ptr_table(wa_list, DEV), ptr_table(wb_list, DEV)
+    tmp_shrink, tmp_expand = sgmv.get_tmp_tensors(len(starts), r, x.device)
+    y_graph = torch.zeros((B, H), dtype=torch.float16, device=DEV)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, pool=None):
+        v = sgmv.lora_a_sgmv_cutlass(x, tmp_shrink, wa_ptr, s_start, s_end, layer, r)
+        sgmv.lora_b_sgmv_cutlass(y_graph, v, tmp_expand, wb_ptr, s_start, s_end, layer)
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.allclose(y_ours, y_graph, rtol=KAT["rtol"], atol=KAT["atol"])
+    for _ in range(2):  # further replays accumulate the same delta again
+        y_graph.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_ours, y_graph)
+
+
+def _ragged_case(dtype, r, h_in, h_out, lens, gen, L=2, gaps=True):
+    """Segments of the given lengths laid out in order with a few uncovered rows between them."""
+    starts, ends, pos = [], [], 0
+    for i, n in enumerate(lens):
+        if gaps and i % 3 == 1:
+            pos += 2  # rows that belong to no segment
+        starts.append(pos)
+        ends.append(pos + n)
+        pos += n
+    T = pos + (3 if gaps else 0)
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    y0 = randn((T, h_out), 0.5, gen, dtype, DEV)
+    a = [randn((L, h_in, r), 0.02, gen, dtype, DEV) if n > 0 else None for n in lens]
+    wa = [stored_sgmv_a(t, r) if t is not None else None for t in a]
+    wb = [randn((L, r, h_out), 0.02, gen, dtype, DEV) if n > 0 else None for n in lens]
+    return T, x, y0, wa, wb, starts, ends
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("r", [8, 16, 32, 64, 128])
+@pytest.mark.parametrize("h_in,h_out,lens", [
+    (4096, 4096, [16, 16, 16, 16]),
+    (1024, 2048, [1, 0, 3, 17, 1, 64, 5, 0, 130]),
+    (4096, 14336, [300, 2, 31, 257]),
+    (14336, 4096, [70, 1, 1, 200]),
+])
+def test_sgmv_shrink_expand_vs_oracle(dtype, r, h_in, h_out, lens):
+    print(f"case dtype={dtype} r={r} h_in={h_in} h_out={h_out} lens={lens}", flush=True)
+    gen = torch.Generator().manual_seed(r * 7 + len(lens))
+    layer = 1
+    T, x, y0, wa, wb, starts, ends = _ragged_case(dtype, r, h_in, h_out, lens, gen)
+    y = y0.clone()
+    v = _run_pair(x, y, wa, wb, starts, ends, layer, r)
+    torch.cuda.synchronize()
+
+    cpu = lambda ts: [t.cpu() if t is not None else None for t in ts]  # noqa: E731
+    v_ref = O.sgmv_ref(torch.zeros((T, r), dtype=dtype), x.cpu(), cpu(wa),
+                       [torch.eye(r, dtype=dtype).expand(2, r, r) if w is not None else None for w in wb],
+                       starts, ends, layer, r)
+    y_ref = O.sgmv_ref(y0.cpu().clone(), x.cpu(), cpu(wa), cpu(wb), starts, ends, layer, r)
+    assert_close(v, v_ref, "shrink output v", max_abs=4e-2)  # |v| reaches 4..8 where one bf16 ulp is 0.031
+    assert_close(y, y_ref, "expand output y")
+    covered = torch.zeros(T, dtype=torch.bool)
+    for s, e in zip(starts, ends):
+        covered[s:e] = True
+    assert torch.equal(y.cpu()[~covered], y0.cpu()[~covered])
+    assert torch.count_nonzero(v.cpu()[~covered]) == 0
+
+
+@pytest.mark.parametrize("r", [48, 80, 96, 112])
+def test_sgmv_other_multiples_of_16(r):
+    """pad_to_min_rank can produce these ranks (punica.py:57-65); the reference's shrink has no
+    instantiation for 48, 80 and 112 (sgmv_config.h:10-15)."""
+    gen = torch.Generator().manual_seed(r)
+    dtype = torch.bfloat16
+    T, x, y0, wa, wb, starts, ends = _ragged_case(dtype, r, 2752, 1152, [40, 3, 129], gen)
+    y = y0.clone()
+    _run_pair(x, y, wa, wb, starts, ends, 0, r)
+    cpu = lambda ts: [t.cpu() if t is not None else None for t in ts]  # noqa: E731
+    y_ref = O.sgmv_ref(y0.cpu().clone(), x.cpu(), cpu(wa), cpu(wb), starts, ends, 0, r)
+    assert_close(y, y_ref, "y")
+
+
+def test_sgmv_empty_negative_and_null_segments_touch_nothing():
+    dtype, r, h = torch.bfloat16, 64, 1024
+    gen = torch.Generator().manual_seed(2)
+    T = 40
+    x = randn((T, h), 1.0, gen, dtype, DEV)
+    y0 = randn((T, h), 0.5, gen, dtype, DEV)
+    wa = stored_sgmv_a(randn((1, h, r), 0.02, gen, dtype, DEV), r)
+    wb = randn((1, r, h), 0.02, gen, dtype, DEV)
+    starts = [0, 10, -1, 20, 30]
+    ends = [10, 10, -1, 15, 40]  # empty, (-1, -1), negative length
+    wa_list = [wa, None, None, None, wa]
+    wb_list = [wb, None, None, None, wb]
+    y = y0.clone()
+    v = _run_pair(x, y, wa_list, wb_list, starts, ends, 0, r)
+    y_ref = O.sgmv_ref(y0.cpu().clone(), x.cpu(), [wa.cpu(), None, None, None, wa.cpu()],
+                       [wb.cpu(), None, None, None, wb.cpu()], starts, ends, 0, r)
+    assert_close(y, y_ref, "y")
+    assert torch.equal(y.cpu()[10:30], y0.cpu()[10:30])
+    assert torch.count_nonzero(v.cpu()[10:30]) == 0
+    # no segment at all
+    y2 = y0.clone()
+    _run_pair(x, y2, [None], [None], [5], [5], 0, r)
+    assert torch.equal(y2, y0)
+
+
+def test_sgmv_routing_is_bit_exact():
+    """Every segment's A picks x[:, 0] = 1 and its B writes (i + 1) / 128 + j / 32 into column j."""
+    dtype, r, h_in, h_out = torch.float16, 16, 512, 128
+    lens = [5, 1, 40, 16, 300, 2]
+    starts, ends, pos = [], [], 3
+    for n in lens:
+        starts.append(pos)
+        ends.append(pos + n)
+        pos += n + 1
+    T = pos
+    x = torch.randn(T, h_in, generator=torch.Generator().manual_seed(0))
+    x[:, 0] = 1.0
+    x = x.to(dtype).to(DEV)
+    wa, wb = [], []
+    for i in range(len(lens)):
+        a = torch.zeros(1, r, h_in)
+        a[0, 0, 0] = 1.0
+        b = torch.zeros(1, r, h_out)
+        b[0, 0, :] = (i + 1) / 128.0 + torch.arange(h_out) / 32.0
+        wa.append(a.to(dtype).to(DEV))
+        wb.append(b.to(dtype).to(DEV))
+    y = torch.full((T, h_out), 0.5, dtype=dtype, device=DEV)
+    _run_pair(x, y, wa, wb, starts, ends, 0, r)
+    expect = torch.full((T, h_out), 0.5)
+    for i, (s, e) in enumerate(zip(starts, ends)):
+        expect[s:e] += (i + 1) / 128.0 + torch.arange(h_out) / 32.0
+    assert torch.equal(y.cpu(), expect.to(dtype))
+
+
+def test_sgmv_expand_column_window():
+    dtype, r, h_in = torch.bfloat16, 32, 4096
+    sizes = [14336, 14336]
+    gen = torch.Generator().manual_seed(4)
+    lens = [33, 100, 7]
+    T, x, _, _, _, starts, ends = _ragged_case(dtype, r, h_in, 8, lens, gen, gaps=False)
+    y0 = randn((T, sum(sizes)), 0.5, gen, dtype, DEV)
+    y = y0.clone()
+    y_ref = y0.cpu().clone()
+    s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
+    off = 0
+    for h_out in sizes:
+        wa = [stored_sgmv_a(randn((1, h_in, r), 0.02, gen, dtype, DEV), r) for _ in lens]
+        wb = [randn((1, r, h_out), 0.02, gen, dtype, DEV) for _ in lens]
+        tmp_shrink, tmp_expand = sgmv.get_tmp_tensors(len(lens), r, x.device)
+        v = sgmv.lora_a_sgmv_cutlass(x, tmp_shrink, ptr_table(wa, DEV), s_start, s_end, 0, r)
+        sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_expand, ptr_table(wb, DEV), s_start, s_end, 0, off, h_out)
+        part = O.sgmv_ref(y_ref[:, off:off + h_out].clone(), x.cpu(), [w.cpu() for w in wa], [w.cpu() for w in wb],
+                          starts, ends, 0, r)
+        y_ref[:, off:off + h_out] = part
+        off += h_out
+    assert_close(y, y_ref, "fused gate/up output")
+
+
+def test_sgmv_split_k_is_deterministic_and_leaves_workspace_clean():
+    """Few row tiles and a long hidden dimension force the split-K path; repeated calls must give
+    bit-identical results (fixed summation order, counters reset by the last arrival)."""
+    dtype, r, h_in = torch.bfloat16, 64, 14336
+    gen = torch.Generator().manual_seed(9)
+    T, x, _, wa, _, starts, ends = _ragged_case(dtype, r, h_in, 8, [16, 5, 48], gen, gaps=True)
+    s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
+    tmp = sgmv.get_tmp_tensor(x.device)
+    outs = [sgmv.lora_a_sgmv_cutlass(x, tmp, ptr_table(wa, DEV), s_start, s_end, 1, r) for _ in range(4)]
+    torch.cuda.synchronize()
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    v_ref = O.sgmv_ref(torch.zeros((T, r), dtype=dtype), x.cpu(), [w.cpu() for w in wa],
+                       [torch.eye(r, dtype=dtype).expand(2, r, r)] * 3, starts, ends, 1, r)
+    assert_close(outs[0], v_ref, "v", max_abs=4e-2)
+
+
+def test_sgmv_errors_raise_runtime_error():
+    x = torch.zeros((4, 1024), dtype=torch.bfloat16, device=DEV)
+    ptr = torch.zeros(1, dtype=torch.int64, device=DEV)
+    s = torch.zeros(1, dtype=torch.int32, device=DEV)
+    good_shrink, good_expand = sgmv.get_tmp_tensors(1, 16, x.device)
+    with pytest.raises(RuntimeError, match="CHECK_EQ"):
+        sgmv.lora_a_sgmv_cutlass(x, good_expand, ptr, s, s, 0, 16)  # 60-byte tmp where 8 MiB is required
+    with pytest.raises(RuntimeError, match="CHECK_EQ"):
+        sgmv.lora_b_sgmv_cutlass(torch.zeros((4, 1024), dtype=torch.bfloat16, device=DEV),
+                                 torch.zeros((4, 16), dtype=torch.bfloat16, device=DEV), good_shrink, ptr, s, s, 0)
+    with pytest.raises(RuntimeError, match="No suitable kernel"):
+        sgmv.lora_a_sgmv_cutlass(x.float(), good_shrink, ptr, s, s, 0, 16)
+    with pytest.raises(RuntimeError, match="int32"):
+        sgmv.lora_a_sgmv_cutlass(x, good_shrink, ptr, s.long(), s.long(), 0, 16)
