@@ -21,6 +21,7 @@ import os
 import statistics
 import sys
 import time
+from collections import defaultdict
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
@@ -37,6 +38,9 @@ def parse_args():
     p.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
     p.add_argument("--layers", type=int, default=0, help="layers per step (0 = the configuration's default)")
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--pattern", choices=["fused", "reference"], default="fused",
+                   help="launch sequence: the one lorax_amd.layers issues, or the reference caller's")
+    p.add_argument("--no-plan", action="store_true", help="fused pattern without the host-built routing plan")
     p.add_argument("--eager", action="store_true", help="launch every step eagerly instead of replaying a graph")
     return p.parse_args()
 
@@ -52,74 +56,120 @@ def build_workload(cfg: int, layers: int, device):
 
 
 class Plan:
-    """Pre-built kernel arguments of one workload: per projection the rank groups' tables plus the
-    static v and y buffers, and closures that issue the zero-fill / shrink / expand launches."""
+    """Pre-built kernel arguments of one workload: per projection group the rank groups' tables plus the
+    static v and y buffers, and closures that issue the launches of ONE layer in order.
 
-    def __init__(self, w):
+    pattern "fused" is what lorax_amd.layers issues: in decode one batched shrink launch and one batched
+    expand launch per projection group and rank (the shrink overwrites v, no zero-fill); in prefill a
+    zero-fill, a shrink and an expand per projection and rank.  pattern "reference" is the reference
+    caller's sequence (utils/layers.py:114-164): zero-fill, shrink, expand for every projection and rank.
+    """
+
+    def __init__(self, w, pattern="fused", use_plan=True):
         import torch
 
         from lorax_amd.adapters import LORA
 
         self.w = w
+        self.use_plan = use_plan
         self.batch = w.batch_data()
-        self.calls = []  # (kind, fn, algorithmic bytes, flops) in issue order for ONE layer; fn(layer)
-        e = 2
+        self.calls = []  # (kind, fn(layer), algorithmic bytes, flops)
         T = w.num_tokens
         for group in w.groups:
             x = w.inputs[group.name]
             y = torch.zeros((T, group.h_out), dtype=w.dtype, device=w.device)
+            jobs = []  # (use_sgmv, r, rank_segments, offset, width)
             off = 0
             for name, size in zip(group.layer_names, group.sizes):
                 data = self.batch.data.get(name, {}).get(LORA)
                 if data is not None:
                     for r, rd in data.rank_data.items():
-                        self._add_rank_group(data.use_sgmv, x, y, off, size, group, r, rd, e)
+                        jobs.append((data.use_sgmv, r, rd, off, size))
                 off += size
+            decode = defaultdict(list)
+            for use_sgmv, r, rd, off, size in jobs:
+                if use_sgmv:
+                    self._add_sgmv(x, y, off, size, group.h_in, r, rd)
+                elif pattern == "reference":
+                    self._add_bgmv_reference(x, y, off, size, group.h_in, r, rd)
+                else:
+                    decode[r].append((rd, off, size))
+            for r, chunk_jobs in decode.items():
+                for i in range(0, len(chunk_jobs), 4):
+                    self._add_bgmv_fused(x, y, group.h_in, r, chunk_jobs[i:i + 4])
 
-    def _add_rank_group(self, use_sgmv, x, y, off, size, group, r, rd, e):
+    @staticmethod
+    def _bgmv_counts(rd):
+        routed = rd.indices >= 0
+        rows = int(routed.sum().item())
+        uniq = len(set(rd.lora_a_ptr[rd.indices[routed]].tolist()))
+        return rows, uniq
+
+    def _add_sgmv(self, x, y, off, size, h_in, r, rd):
         import torch
 
         from lorax_amd import sgmv
 
-        T = x.size(0)
-        v = torch.zeros((T, r), dtype=x.dtype, device=x.device)
-        if use_sgmv:
-            lens = (rd.segment_ends - rd.segment_starts).clamp(min=0)
-            rows = int(lens.sum().item())
-            uniq = len(set(rd.lora_a_ptr[lens > 0].tolist()))
-            starts, ends, tmp_s, tmp_e = rd.segment_starts, rd.segment_ends, rd.tmp_shrink, rd.tmp_expand
-            a_ptr, b_ptr = rd.lora_a_ptr, rd.lora_b_ptr
-            a_is_rh = not sgmv.use_cutlass_shrink(r)
+        e = 2
+        v = torch.zeros((x.size(0), r), dtype=x.dtype, device=x.device)
+        lens = (rd.segment_ends - rd.segment_starts).clamp(min=0)
+        rows = int(lens.sum().item())
+        uniq = len(set(rd.lora_a_ptr[lens > 0].tolist()))
+        starts, ends, tmp_s, tmp_e = rd.segment_starts, rd.segment_ends, rd.tmp_shrink, rd.tmp_expand
+        a_ptr, b_ptr = rd.lora_a_ptr, rd.lora_b_ptr
+        a_is_rh = not sgmv.use_cutlass_shrink(r)
 
-            def shrink(layer):
-                if a_is_rh:
-                    sgmv._kernels.sgmv_shrink(v, x, a_ptr, starts, ends, tmp_s, layer)
-                else:
-                    sgmv._kernels.sgmv_cutlass(v, x, a_ptr, starts, ends, tmp_s, layer)
+        def shrink(layer):
+            if a_is_rh:
+                sgmv._kernels.sgmv_shrink(v, x, a_ptr, starts, ends, tmp_s, layer)
+            else:
+                sgmv._kernels.sgmv_cutlass(v, x, a_ptr, starts, ends, tmp_s, layer)
 
-            def expand(layer):
-                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_ptr, starts, ends, layer, off, size)
+        def expand(layer):
+            sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_ptr, starts, ends, layer, off, size)
 
-            kind = "sgmv"
-        else:
-            routed = rd.indices >= 0
-            rows = int(routed.sum().item())
-            uniq = len(set(rd.lora_a_ptr[rd.indices[routed]].tolist()))
-            idx, a_ptr, b_ptr = rd.indices, rd.lora_a_ptr, rd.lora_b_ptr
-
-            def shrink(layer):
-                sgmv.add_lora_a_bgmv(v, x, a_ptr, idx, layer)
-
-            def expand(layer):
-                sgmv.add_lora_b_bgmv_slice(y, v, b_ptr, idx, layer, off, size)
-
-            kind = "bgmv"
-        h_in = group.h_in
-        shrink_bytes = rows * h_in * e + uniq * r * h_in * e + rows * r * e
-        expand_bytes = rows * r * e + uniq * r * size * e + 2 * rows * size * e
         self.calls.append(("zero", lambda layer: v.zero_(), 0, 0))
-        self.calls.append((f"{kind}_shrink", shrink, shrink_bytes, 2 * rows * r * h_in))
-        self.calls.append((f"{kind}_expand", expand, expand_bytes, 2 * rows * r * size))
+        self.calls.append(("sgmv_shrink", shrink, rows * h_in * e + uniq * r * h_in * e + rows * r * e,
+                           2 * rows * r * h_in))
+        self.calls.append(("sgmv_expand", expand, rows * r * e + uniq * r * size * e + 2 * rows * size * e,
+                           2 * rows * r * size))
+
+    def _add_bgmv_reference(self, x, y, off, size, h_in, r, rd):
+        import torch
+
+        from lorax_amd import sgmv
+
+        e = 2
+        v = torch.zeros((x.size(0), r), dtype=x.dtype, device=x.device)
+        rows, uniq = self._bgmv_counts(rd)
+        idx, a_ptr, b_ptr = rd.indices, rd.lora_a_ptr, rd.lora_b_ptr
+        self.calls.append(("zero", lambda layer: v.zero_(), 0, 0))
+        self.calls.append(("bgmv_shrink", lambda layer: sgmv.add_lora_a_bgmv(v, x, a_ptr, idx, layer),
+                           rows * h_in * e + uniq * r * h_in * e + rows * r * e, 2 * rows * r * h_in))
+        self.calls.append(("bgmv_expand",
+                           lambda layer: sgmv.add_lora_b_bgmv_slice(y, v, b_ptr, idx, layer, off, size),
+                           rows * r * e + uniq * r * size * e + 2 * rows * size * e, 2 * rows * r * size))
+
+    def _add_bgmv_fused(self, x, y, h_in, r, jobs):
+        import torch
+
+        from lorax_amd import _native
+
+        e = 2
+        vs = torch.zeros((len(jobs), x.size(0), r), dtype=x.dtype, device=x.device).unbind(0)
+        shrink_problems = [(v, x, rd.lora_a_ptr, rd.indices, 0, None) for v, (rd, _, _) in zip(vs, jobs)]
+        expand_problems = [(y, v, rd.lora_b_ptr, rd.indices, off, size) for v, (rd, off, size) in zip(vs, jobs)]
+        counts = [self._bgmv_counts(rd) for rd, _, _ in jobs]
+        any_routed = torch.stack([rd.indices >= 0 for rd, _, _ in jobs]).any(0)
+        x_rows = int(any_routed.sum().item())  # the shared input is read once per launch
+        shrink_bytes = x_rows * h_in * e + sum(u * r * h_in * e + n * r * e for n, u in counts)
+        expand_bytes = sum(n * r * e + u * r * size * e + 2 * n * size * e
+                           for (n, u), (_, _, size) in zip(counts, jobs))
+        plans = [rd.plan for rd, _, _ in jobs] if self.use_plan else None
+        self.calls.append(("bgmv_shrink", lambda layer: _native.bgmv_multi(shrink_problems, layer, 1.0, False, plans),
+                           shrink_bytes, sum(2 * n * r * h_in for n, _ in counts)))
+        self.calls.append(("bgmv_expand", lambda layer: _native.bgmv_multi(expand_problems, layer, 1.0, True, plans),
+                           expand_bytes, sum(2 * n * r * size for (n, _), (_, _, size) in zip(counts, jobs))))
 
     def issue(self, layers, kinds=None):
         n = 0
@@ -133,8 +183,8 @@ class Plan:
     def bytes_per_layer(self, kind=None):
         return sum(b for k, _, b, _ in self.calls if kind is None or k == kind)
 
-    def launches_per_layer(self, kind):
-        return sum(1 for k, _, _, _ in self.calls if k == kind)
+    def launches_per_layer(self, kind=None):
+        return sum(1 for k, _, _, _ in self.calls if kind is None or k == kind)
 
 
 def capture(plan, layers, kinds=None):
@@ -244,7 +294,7 @@ def main():
 
     w = build_workload(args.config, args.layers, device)
     L = w.num_layers
-    plan = Plan(w)
+    plan = Plan(w, args.pattern, not args.no_plan)
     torch.cuda.synchronize()
 
     if args.eager:
@@ -309,6 +359,8 @@ def main():
             "layers_per_step": L,
             "projections": [n for g in w.groups for n in g.layer_names],
             "launch": "eager" if args.eager else "hip_graph",
+            "pattern": args.pattern,
+            "launches_per_layer": plan.launches_per_layer(),
             "algorithmic_bytes_per_layer": plan.bytes_per_layer(),
             "step_GBps": plan.bytes_per_layer() * L / (elapsed / args.steps) / 1e9,
         },

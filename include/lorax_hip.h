@@ -72,6 +72,46 @@ int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* ind
                int64_t y_stride, int64_t layer_idx, float scale, int32_t dtype, void* stream);
 
 /*
+ * Several BGMV problems in one launch.  No counterpart in the reference, whose caller issues
+ * one dispatch_bgmv per projection and rank group (lorax_server/utils/layers.py:143-164); it
+ * exists because a decode-size BGMV is shorter than a launch, so the projections that share an
+ * input (q/k/v, gate/up) are better issued together.
+ *
+ * `problems` is a HOST array of `num_problems` (<= 4) descriptors; the pointers inside are
+ * device pointers.  All problems share num_tokens, h_in, layer_idx, scale, dtype, the direction
+ * (h_in < h_out means expand) and the LoRA rank; expand problems may differ in h_out.  Each
+ * problem is computed exactly as by lorax_bgmv.  accumulate = 0 (shrink launches only) stores
+ * dtype(sum) instead of adding it, so the caller need not zero v first; rows of tokens whose
+ * index is negative are not written in either mode.
+ *
+ * Routing plan (optional).  Finding which tokens share an adapter costs every workgroup a scan
+ * of indices[]; a caller that builds the index tables on the host anyway (as the reference does,
+ * lorax_server/adapters/lora.py:354-375) can hand over the result instead: `plan` points to
+ * num_groups records of 8 int64 in device memory,
+ *   [0] number of tokens in the chunk (1..4)   [1..4] their row numbers (unused ones repeat [1])
+ *   [5] device address of the adapter's A stack [L, r, h_in]  (read by shrink launches)
+ *   [6] device address of the adapter's B^T stack [L, h_out, r] (read by expand launches)
+ *   [7] reserved
+ * where every chunk holds tokens of ONE adapter and every routed token is in exactly one chunk.
+ * With a plan, w_ptrs and indices are not read and may be NULL.
+ */
+typedef struct lorax_bgmv_problem {
+  void* y;                /* [num_tokens, y_stride] output                         */
+  const void* x;          /* [num_tokens, h_in] input                              */
+  const int64_t* w_ptrs;  /* device addresses of the adapters' [L, h_out, h_in] stacks */
+  const int64_t* indices; /* [num_tokens] index into w_ptrs, negative = no adapter */
+  int64_t y_offset;       /* first output column inside a row of y                 */
+  int64_t y_stride;       /* row pitch of y in elements                            */
+  int32_t h_out;
+  const int64_t* plan;    /* optional routing plan (see above), else NULL          */
+  int32_t num_groups;     /* records in plan                                       */
+} lorax_bgmv_problem_t;
+
+int lorax_bgmv_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems, int64_t num_tokens,
+                     int32_t h_in, int64_t layer_idx, float scale, int32_t accumulate, int32_t dtype,
+                     void* stream);
+
+/*
  * SGMV shrink.  Replaces sgmv_shrink (punica_ops.cc:369-411,
  * sgmv_flashinfer/sgmv_all.cu:10-65) for a_layout = LORAX_A_RH and the shrink
  * direction of sgmv_cutlass (punica_ops.cc:338-367, sgmv/sgmv_cutlass.cuh:132-178)

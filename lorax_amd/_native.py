@@ -22,11 +22,36 @@ A_RH, A_HR = 0, 1
 SHRINK_TMP_BYTES = 8 * 1024 * 1024
 
 _c = ctypes
+
+
+class BgmvProblem(ctypes.Structure):
+    """lorax_bgmv_problem_t of include/lorax_hip.h."""
+
+    _fields_ = [
+        ("y", _c.c_void_p),
+        ("x", _c.c_void_p),
+        ("w_ptrs", _c.c_void_p),
+        ("indices", _c.c_void_p),
+        ("y_offset", _c.c_int64),
+        ("y_stride", _c.c_int64),
+        ("h_out", _c.c_int32),
+        ("plan", _c.c_void_p),
+        ("num_groups", _c.c_int32),
+    ]
+
+
+MAX_BGMV_PROBLEMS = 4
+
 _SIGNATURES = {
     "lorax_bgmv": (
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int32, _c.c_int32,
          _c.c_int64, _c.c_int64, _c.c_int64, _c.c_float, _c.c_int32, _c.c_void_p],
+    ),
+    "lorax_bgmv_multi": (
+        _c.c_int,
+        [_c.POINTER(BgmvProblem), _c.c_int32, _c.c_int64, _c.c_int32, _c.c_int64, _c.c_float, _c.c_int32,
+         _c.c_int32, _c.c_void_p],
     ),
     "lorax_sgmv_shrink": (
         _c.c_int,
@@ -170,6 +195,51 @@ def bgmv(y, x, w_ptr, indicies, layer_idx, scale, y_offset=0, y_slice_size=None)
             y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), indicies.data_ptr(), x.size(0), x.size(1), h_out,
             int(y_offset), y.size(1), int(layer_idx), float(scale), _dtype_code(x), _stream(x),
         )
+    if rc != 0:
+        _raise_last(rc)
+
+
+PLAN_RECORD_WORDS = 8
+
+
+def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> None:
+    """lorax_bgmv_multi: `problems` is a list of up to 4 tuples (y, x, w_ptr, indicies, y_offset, y_slice_size)
+    that share x.shape, the direction and the rank; y_slice_size None means the whole width of y.
+    `plans`, if given, holds one routing plan per problem: an int64 device tensor [num_groups, 8]."""
+    if not 1 <= len(problems) <= MAX_BGMV_PROBLEMS:
+        raise RuntimeError(f"between 1 and {MAX_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
+    arr = (BgmvProblem * len(problems))()
+    x0 = problems[0][1]
+    for i, (y, x, w_ptr, indicies, y_offset, y_slice_size) in enumerate(problems):
+        _check_input(y, "y", 2)
+        _check_input(x, "x", 2)
+        _check_input(w_ptr, "w_ptr", 1)
+        _check_input(indicies, "indicies", 1)
+        _check_same(y, x, w_ptr, indicies)
+        if w_ptr.dtype != torch.int64 or indicies.dtype != torch.int64:
+            raise RuntimeError("w_ptr and indicies must be int64 tensors")
+        if x.shape != x0.shape or x.dtype != x0.dtype or x.device != x0.device:
+            raise RuntimeError("all problems of one launch must have inputs of one shape, dtype and device")
+        if indicies.size(0) != x.size(0) or y.size(0) != x.size(0):
+            raise RuntimeError(
+                f"CHECK_EQ(indicies.size(0), x.size(0)) / CHECK_EQ(y.size(0), x.size(0)) failed. "
+                f"{indicies.size(0)}, {y.size(0)} vs {x.size(0)}"
+            )
+        h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
+        plan_ptr, num_groups = None, 0
+        if plans is not None:
+            plan = plans[i]
+            _check_input(plan, "plan", 2)
+            if plan.dtype != torch.int64 or plan.size(1) != PLAN_RECORD_WORDS or plan.device != x.device:
+                raise RuntimeError(f"plan must be an int64 [num_groups, {PLAN_RECORD_WORDS}] tensor on the device of x")
+            plan_ptr, num_groups = plan.data_ptr(), plan.size(0)
+            if num_groups == 0:
+                plan_ptr = x.data_ptr()  # an empty plan has no storage; any non-null address will do
+        arr[i] = BgmvProblem(y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), indicies.data_ptr(), int(y_offset),
+                             y.size(1), h_out, plan_ptr, num_groups)
+    with torch.cuda.device(x0.device):
+        rc = lib().lorax_bgmv_multi(arr, len(problems), x0.size(0), x0.size(1), int(layer_idx), float(scale),
+                                    1 if accumulate else 0, _dtype_code(x0), _stream(x0))
     if rc != 0:
         _raise_last(rc)
 

@@ -172,6 +172,32 @@ class RankSegments:
     segment_ends: Optional[torch.Tensor]
     # decode (BGMV)
     indices: Optional[torch.Tensor]
+    # decode: routing plan for the batched BGMV launches, int64 [num_chunks, 8] on the device; one record
+    # per chunk of up to BGMV_PLAN_GROUP tokens of one adapter: [count, tok0..tok3, address of the A stack,
+    # address of the B^T stack, 0]. Derived from `indices` and the pointer tables; no counterpart in the
+    # reference, whose kernels take one token per thread block.
+    plan: Optional[torch.Tensor] = None
+
+
+BGMV_PLAN_GROUP = 4
+BGMV_PLAN_WORDS = 8
+
+
+def build_bgmv_plan(token_slots: List[int], a_addrs: List[int], b_addrs: List[int]) -> List[List[int]]:
+    """Cuts the tokens of every adapter slot, in token order, into chunks of at most BGMV_PLAN_GROUP and
+    returns one plan record per chunk. token_slots[t] is the token's index into the rank group's pointer
+    slice (-1 = not in the group); a_addrs / b_addrs are the addresses in that slice."""
+    by_slot: Dict[int, List[int]] = {}
+    for t, s in enumerate(token_slots):
+        if s >= 0:
+            by_slot.setdefault(s, []).append(t)
+    records = []
+    for s, toks in by_slot.items():
+        for i in range(0, len(toks), BGMV_PLAN_GROUP):
+            chunk = toks[i : i + BGMV_PLAN_GROUP]
+            pad = [chunk[0]] * (BGMV_PLAN_GROUP - len(chunk))
+            records.append([len(chunk), *chunk, *pad, a_addrs[s], b_addrs[s], 0])
+    return records
 
 
 def _unwrap(weights):
@@ -264,7 +290,7 @@ class BatchLoraWeights(BatchAdapterWeights):
         token_adapters = None if use_sgmv else meta.adapter_indices.tolist()
         rank_data: Dict[int, RankSegments] = {}
         for rank, segs in by_rank.items():
-            tmp_shrink = tmp_expand = starts = ends = token_slots = None
+            tmp_shrink = tmp_expand = starts = ends = token_slots = plan = None
             if use_sgmv:
                 tmp_shrink, tmp_expand = get_tmp_tensors(len(segs), rank, device)
                 starts = meta.adapter_segments[segs]
@@ -278,11 +304,10 @@ class BatchLoraWeights(BatchAdapterWeights):
                 slot: Dict[int, int] = {}
                 for pos, s in enumerate(segs):
                     slot.setdefault(seg_adapters[s], pos)
-                token_slots = torch.tensor(
-                    [slot.get(a, -1) if (a in loras and loras[a].lora_a_r == rank) else -1 for a in token_adapters],
-                    dtype=torch.int64,
-                    device=device,
-                )
+                slots = [slot.get(a, -1) if (a in loras and loras[a].lora_a_r == rank) else -1 for a in token_adapters]
+                token_slots = torch.tensor(slots, dtype=torch.int64, device=device)
+                records = build_bgmv_plan(slots, [a_addr[s] for s in segs], [b_addr[s] for s in segs])
+                plan = torch.tensor(records, dtype=torch.int64, device=device).reshape(-1, BGMV_PLAN_WORDS)
             rank_data[rank] = RankSegments(
                 rank=rank,
                 lora_a_ptr=lora_a_ptr[segs],
@@ -292,6 +317,7 @@ class BatchLoraWeights(BatchAdapterWeights):
                 segment_starts=starts,
                 segment_ends=ends,
                 indices=token_slots,
+                plan=plan,
             )
 
         return cls(

@@ -32,16 +32,33 @@ __device__ __forceinline__ void bgmv_shrink_body(typename D::E* __restrict__ Y,
                                                  const typename D::E* __restrict__ A,
                                                  const int (&toks)[kGroup], int h_in, int row0,
                                                  int64_t y_offset, int64_t y_stride, float scale,
-                                                 float* red) {
+                                                 bool accumulate_into_y, float* red) {
   using vec8 = typename D::vec8;
+  using E = typename D::E;
   const int tid = threadIdx.x;
+
+  // The thread that will write output (j, g) fetches the old value now, so that the
+  // read-modify-write at the end does not add a memory round trip.
+  E* yp = nullptr;
+  E y_old = static_cast<E>(0.f);
+  if (tid < RS * NT) {
+    const int j = tid / NT;
+    const int g = tid % NT;
+    int tok = toks[0];
+#pragma unroll
+    for (int q = 1; q < NT; ++q)
+      if (g == q) tok = toks[q];
+    yp = Y + static_cast<int64_t>(tok) * y_stride + y_offset + row0 + j;
+    if (accumulate_into_y) y_old = *yp;
+  }
+
   float acc[RS][NT];
 #pragma unroll
   for (int j = 0; j < RS; ++j)
 #pragma unroll
     for (int g = 0; g < NT; ++g) acc[j][g] = 0.f;
 
-  const typename D::E* xrow[NT];
+  const E* xrow[NT];
 #pragma unroll
   for (int g = 0; g < NT; ++g) xrow[g] = X + static_cast<int64_t>(toks[g]) * h_in;
 
@@ -87,44 +104,61 @@ __device__ __forceinline__ void bgmv_shrink_body(typename D::E* __restrict__ Y,
     float s = 0.f;
 #pragma unroll
     for (int w = 0; w < kBgmvThreads / kWave; ++w) s += red[w * NV + tid];
-    const int j = tid / NT;
-    const int g = tid % NT;
-    int tok = toks[0];
-#pragma unroll
-    for (int q = 1; q < NT; ++q)
-      if (g == q) tok = toks[q];
-    typename D::E* yp = Y + static_cast<int64_t>(tok) * y_stride + y_offset + row0 + j;
-    *yp = accumulate<D>(*yp, s * scale);
+    *yp = accumulate<D>(y_old, s * scale);
   }
+}
+
+// Resolves the token chunk of workgroup row blockIdx.y and the address of its adapter's stack.
+// With a routing plan (built once per batch next to the index tables) this is one 64-byte
+// record: [ntok, tok0..tok3, address of the A stack, address of the B^T stack, reserved];
+// without one, the chunk is found by scanning indices[] (group_tokens).  Returns the number of
+// tokens, 0 if the workgroup has nothing to do.  Wave-uniform.
+__device__ __forceinline__ int resolve_chunk(const BgmvProblem& P, int num_tokens, bool expand,
+                                             int (&toks)[kGroup], int64_t& stack_addr) {
+  if (P.plan != nullptr) {
+    if (static_cast<int>(blockIdx.y) >= P.num_groups) return 0;
+    const int64_t* rec = P.plan + static_cast<int64_t>(blockIdx.y) * kPlanRecordWords;
+    const int n = static_cast<int>(rec[0]);
+#pragma unroll
+    for (int g = 0; g < kGroup; ++g) toks[g] = static_cast<int>(rec[1 + g]);
+    stack_addr = rec[expand ? 6 : 5];
+    return n;
+  }
+  int64_t idx;
+  const int n = group_tokens<kGroup>(P.indices, num_tokens, blockIdx.y, idx, toks);
+  if (n == 0) return 0;
+  stack_addr = P.w_ptrs[idx];
+  return n;
 }
 
 template <typename D, int RS>
 __global__ __launch_bounds__(kBgmvThreads) void bgmv_shrink_kernel(
-    typename D::E* __restrict__ Y, const typename D::E* __restrict__ X,
-    const int64_t* __restrict__ W, const int64_t* __restrict__ indices, int num_tokens, int h_in,
-    int r, int64_t y_offset, int64_t y_stride, int64_t layer_idx, float scale) {
+    const BgmvBatch batch, int num_tokens, int h_in, int r, int64_t layer_idx, float scale,
+    int accumulate_into_y) {
   __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<RS * kGroup>::value];
-  const int b = blockIdx.y;
-  const int64_t idx = indices[b];
-  if (idx < 0) return;
+  using E = typename D::E;
+  const BgmvProblem& P = batch.p[blockIdx.z];
   int toks[kGroup];
-  const int n = group_tokens<kGroup>(indices, num_tokens, b, idx, toks);
+  int64_t stack_addr;
+  const int n = resolve_chunk(P, num_tokens, false, toks, stack_addr);
   if (n == 0) return;
   const int row0 = blockIdx.x * RS;
-  const typename D::E* A = reinterpret_cast<const typename D::E*>(W[idx]) +
-                           (layer_idx * r + row0) * static_cast<int64_t>(h_in);
+  const E* A = reinterpret_cast<const E*>(stack_addr) + (layer_idx * r + row0) * static_cast<int64_t>(h_in);
+  E* Y = static_cast<E*>(P.y);
+  const E* X = static_cast<const E*>(P.x);
+  const bool acc_y = accumulate_into_y != 0;
   switch (n) {
     case 1:
-      bgmv_shrink_body<D, RS, 1>(Y, X, A, toks, h_in, row0, y_offset, y_stride, scale, red);
+      bgmv_shrink_body<D, RS, 1>(Y, X, A, toks, h_in, row0, P.y_offset, P.y_stride, scale, acc_y, red);
       break;
     case 2:
-      bgmv_shrink_body<D, RS, 2>(Y, X, A, toks, h_in, row0, y_offset, y_stride, scale, red);
+      bgmv_shrink_body<D, RS, 2>(Y, X, A, toks, h_in, row0, P.y_offset, P.y_stride, scale, acc_y, red);
       break;
     case 3:
-      bgmv_shrink_body<D, RS, 3>(Y, X, A, toks, h_in, row0, y_offset, y_stride, scale, red);
+      bgmv_shrink_body<D, RS, 3>(Y, X, A, toks, h_in, row0, P.y_offset, P.y_stride, scale, acc_y, red);
       break;
     default:
-      bgmv_shrink_body<D, RS, 4>(Y, X, A, toks, h_in, row0, y_offset, y_stride, scale, red);
+      bgmv_shrink_body<D, RS, 4>(Y, X, A, toks, h_in, row0, P.y_offset, P.y_stride, scale, acc_y, red);
       break;
   }
 }
@@ -200,31 +234,33 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
 }
 
 template <typename D, int CP, int U>
-__global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(
-    typename D::E* __restrict__ Y, const typename D::E* __restrict__ V,
-    const int64_t* __restrict__ W, const int64_t* __restrict__ indices, int num_tokens, int r,
-    int h_out, int64_t y_offset, int64_t y_stride, int64_t layer_idx, float scale) {
-  const int b = blockIdx.y;
-  const int64_t idx = indices[b];
-  if (idx < 0) return;
-  int toks[kGroup];
-  const int n = group_tokens<kGroup>(indices, num_tokens, b, idx, toks);
-  if (n == 0) return;
+__global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBatch batch,
+                                                                   int num_tokens, int r,
+                                                                   int64_t layer_idx, float scale) {
+  using E = typename D::E;
+  const BgmvProblem& P = batch.p[blockIdx.z];
+  const int h_out = P.width;
   const int col0 = blockIdx.x * (kBgmvThreads / CP) * U;
-  const typename D::E* B =
-      reinterpret_cast<const typename D::E*>(W[idx]) + layer_idx * h_out * static_cast<int64_t>(r);
+  if (col0 >= h_out) return;  // problems of one batch may differ in width
+  int toks[kGroup];
+  int64_t stack_addr;
+  const int n = resolve_chunk(P, num_tokens, true, toks, stack_addr);
+  if (n == 0) return;
+  const E* B = reinterpret_cast<const E*>(stack_addr) + layer_idx * h_out * static_cast<int64_t>(r);
+  E* Y = static_cast<E*>(P.y);
+  const E* V = static_cast<const E*>(P.x);
   switch (n) {
     case 1:
-      bgmv_expand_body<D, CP, U, 1>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale);
+      bgmv_expand_body<D, CP, U, 1>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
       break;
     case 2:
-      bgmv_expand_body<D, CP, U, 2>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale);
+      bgmv_expand_body<D, CP, U, 2>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
       break;
     case 3:
-      bgmv_expand_body<D, CP, U, 3>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale);
+      bgmv_expand_body<D, CP, U, 3>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
       break;
     default:
-      bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale);
+      bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
       break;
   }
 }
@@ -234,11 +270,10 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(
 // ---------------------------------------------------------------------------------
 template <typename D, int RS>
 static hipError_t launch_shrink_rs(const BgmvArgs& a, hipStream_t stream) {
-  dim3 grid(a.h_out / RS, static_cast<unsigned>(a.num_tokens));
-  hipLaunchKernelGGL((bgmv_shrink_kernel<D, RS>), grid, dim3(kBgmvThreads), 0, stream,
-                     static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x),
-                     a.w_ptrs, a.indices, static_cast<int>(a.num_tokens), a.h_in, a.h_out,
-                     a.y_offset, a.y_stride, a.layer_idx, a.scale);
+  dim3 grid(a.narrow / RS, static_cast<unsigned>(a.grid_rows), a.count);
+  hipLaunchKernelGGL((bgmv_shrink_kernel<D, RS>), grid, dim3(kBgmvThreads), 0, stream, a.batch,
+                     static_cast<int>(a.num_tokens), a.wide_max, a.narrow, a.layer_idx, a.scale,
+                     a.accumulate);
   return hipGetLastError();
 }
 
@@ -246,7 +281,7 @@ template <typename D>
 static hipError_t launch_shrink(const BgmvArgs& a, hipStream_t stream) {
   // Rows per workgroup: 8 when the grid is large enough to fill 256 CUs several times
   // over, fewer rows (more workgroups) for small batches.
-  const int64_t wgs8 = a.num_tokens * (a.h_out / 8);
+  const int64_t wgs8 = a.work_rows * (a.narrow / 8) * a.count;
   int rs = wgs8 >= 2048 ? 8 : (wgs8 >= 512 ? 4 : 2);
   if (tuning().bgmv_shrink_rows > 0) rs = tuning().bgmv_shrink_rows;
   switch (rs) {
@@ -263,17 +298,16 @@ template <typename D, int CP>
 static hipError_t launch_expand_cp(const BgmvArgs& a, hipStream_t stream) {
   constexpr int U = 4;
   constexpr int cols_per_wg = (kBgmvThreads / CP) * U;
-  dim3 grid((a.h_out + cols_per_wg - 1) / cols_per_wg, static_cast<unsigned>(a.num_tokens));
-  hipLaunchKernelGGL((bgmv_expand_kernel<D, CP, U>), grid, dim3(kBgmvThreads), 0, stream,
-                     static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x),
-                     a.w_ptrs, a.indices, static_cast<int>(a.num_tokens), a.h_in, a.h_out,
-                     a.y_offset, a.y_stride, a.layer_idx, a.scale);
+  dim3 grid((a.wide_max + cols_per_wg - 1) / cols_per_wg, static_cast<unsigned>(a.grid_rows),
+            a.count);
+  hipLaunchKernelGGL((bgmv_expand_kernel<D, CP, U>), grid, dim3(kBgmvThreads), 0, stream, a.batch,
+                     static_cast<int>(a.num_tokens), a.narrow, a.layer_idx, a.scale);
   return hipGetLastError();
 }
 
 template <typename D>
 static hipError_t launch_expand(const BgmvArgs& a, hipStream_t stream) {
-  const int chunks = a.h_in / 8;
+  const int chunks = a.narrow / 8;
   if (chunks <= 1) return launch_expand_cp<D, 1>(a, stream);
   if (chunks <= 2) return launch_expand_cp<D, 2>(a, stream);
   if (chunks <= 4) return launch_expand_cp<D, 4>(a, stream);
@@ -282,10 +316,9 @@ static hipError_t launch_expand(const BgmvArgs& a, hipStream_t stream) {
 }
 
 hipError_t launch_bgmv(const BgmvArgs& a, hipStream_t stream) {
-  const bool expand = a.h_in < a.h_out;  // bgmv_impl.cuh:204
   if (a.dtype == LORAX_F16)
-    return expand ? launch_expand<F16>(a, stream) : launch_shrink<F16>(a, stream);
-  return expand ? launch_expand<BF16>(a, stream) : launch_shrink<BF16>(a, stream);
+    return a.expand ? launch_expand<F16>(a, stream) : launch_shrink<F16>(a, stream);
+  return a.expand ? launch_expand<BF16>(a, stream) : launch_shrink<BF16>(a, stream);
 }
 
 }  // namespace lorax

@@ -102,33 +102,89 @@ const Tuning& tuning() {
 
 using namespace lorax;
 
+namespace {
+
+// Validates one batch of BGMV problems that share num_tokens, h_in, direction and layer and
+// launches it.  h_out[i] is problem i's output width.
+int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_tokens, int32_t h_in,
+               int64_t layer_idx, float scale, int32_t accumulate, int32_t dtype, void* stream) {
+  if (count < 0 || count > kMaxBgmvProblems)
+    return fail(LORAX_EINVAL, "num_problems=%d (at most %d per launch)", count, kMaxBgmvProblems);
+  if (num_tokens < 0) return fail(LORAX_EINVAL, "num_tokens=%lld is negative", (long long)num_tokens);
+  if (count == 0 || num_tokens == 0) return LORAX_OK;
+  if (problems == nullptr) return fail(LORAX_EINVAL, "null pointer argument (problems)");
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  BgmvArgs a{};
+  a.count = count;
+  a.expand = h_in < problems[0].h_out;  // bgmv_impl.cuh:204
+  a.narrow = a.expand ? h_in : problems[0].h_out;
+  a.wide_max = a.expand ? 0 : h_in;
+  a.num_tokens = num_tokens;
+  a.layer_idx = layer_idx;
+  a.scale = scale;
+  a.accumulate = accumulate;
+  a.dtype = dtype;
+  const bool planned = problems[0].plan != nullptr;
+  for (int i = 0; i < count; ++i) {
+    const lorax_bgmv_problem_t& q = problems[i];
+    if ((q.plan != nullptr) != planned)
+      return fail(LORAX_EINVAL, "problems of one launch must all carry a plan or none");
+    if (planned) {
+      if (int rc = check_common(q.y, q.x, q.plan, dtype)) return rc;
+      if (q.num_groups < 0 || q.num_groups > 65535)
+        return fail(LORAX_EINVAL, "num_groups=%d out of range", q.num_groups);
+      if (q.num_groups > a.grid_rows) a.grid_rows = q.num_groups;
+    } else {
+      if (int rc = check_common(q.y, q.x, q.w_ptrs, dtype)) return rc;
+      if (q.indices == nullptr) return fail(LORAX_EINVAL, "null pointer argument (indices)");
+    }
+    const int h_out = q.h_out;
+    const bool expand = h_in < h_out;
+    const int narrow = expand ? h_in : h_out;
+    const int wide = expand ? h_out : h_in;
+    // punica_ops.cc:310 (dims < 65536) and bgmv_config.h:12-86 (narrow side 8..128).
+    if (h_in <= 0 || h_out <= 0 || h_in >= 65536 || h_out >= 65536 || narrow % 8 != 0 ||
+        narrow > kMaxRank || wide % 8 != 0)
+      return fail(LORAX_ENOKERNEL, "No suitable kernel. h_in=%d h_out=%d dtype=%d", h_in, h_out, dtype);
+    if (expand != a.expand || narrow != a.narrow)
+      return fail(LORAX_EINVAL, "problems of one launch must share direction and rank (problem %d: h_out=%d)",
+                  i, h_out);
+    if (q.y_offset < 0 || q.y_stride < q.y_offset + h_out)
+      return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld do not hold h_out=%d columns",
+                  (long long)q.y_offset, (long long)q.y_stride, h_out);
+    if (a.expand && h_out > a.wide_max) a.wide_max = h_out;
+    a.batch.p[i] = BgmvProblem{q.y, q.x, q.w_ptrs, q.indices, q.y_offset, q.y_stride, h_out, q.plan, q.num_groups};
+  }
+  if (!planned) a.grid_rows = num_tokens;
+  a.work_rows = planned ? a.grid_rows : (num_tokens + 1) / 2;
+  if (a.grid_rows == 0) return LORAX_OK;
+  if (!a.expand && accumulate != 0 && accumulate != 1)
+    return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
+  if (a.expand && accumulate != 1)
+    return fail(LORAX_EINVAL, "an expand launch always adds to y (accumulate must be 1)");
+  if (num_tokens > 65535)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. num_tokens=%lld exceeds 65535", (long long)num_tokens);
+  const hipError_t e = launch_bgmv(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* indices,
                int64_t num_tokens, int32_t h_in, int32_t h_out, int64_t y_offset,
                int64_t y_stride, int64_t layer_idx, float scale, int32_t dtype, void* stream) {
-  if (num_tokens < 0) return fail(LORAX_EINVAL, "num_tokens=%lld is negative", (long long)num_tokens);
   if (num_tokens == 0) return LORAX_OK;
-  if (int rc = check_common(y, x, w_ptrs, dtype)) return rc;
-  if (indices == nullptr) return fail(LORAX_EINVAL, "null pointer argument (indices)");
-  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
-  const bool expand = h_in < h_out;
-  const int narrow = expand ? h_in : h_out;
-  const int wide = expand ? h_out : h_in;
-  // punica_ops.cc:310 (dims < 65536) and bgmv_config.h:12-86 (narrow side 8..128).
-  if (h_in <= 0 || h_out <= 0 || h_in >= 65536 || h_out >= 65536 || narrow % 8 != 0 ||
-      narrow > kMaxRank || wide % 8 != 0)
-    return fail(LORAX_ENOKERNEL, "No suitable kernel. h_in=%d h_out=%d dtype=%d", h_in, h_out, dtype);
-  if (num_tokens > 65535)
-    return fail(LORAX_ENOKERNEL, "No suitable kernel. num_tokens=%lld exceeds 65535",
-                (long long)num_tokens);
-  if (y_offset < 0 || y_stride < y_offset + h_out)
-    return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld do not hold h_out=%d columns",
-                (long long)y_offset, (long long)y_stride, h_out);
-  BgmvArgs a{y, x, w_ptrs, indices, num_tokens, h_in, h_out, y_offset, y_stride, layer_idx, scale, dtype};
-  const hipError_t e = launch_bgmv(a, static_cast<hipStream_t>(stream));
-  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString(e));
-  return LORAX_OK;
+  const lorax_bgmv_problem_t one{y, x, w_ptrs, indices, y_offset, y_stride, h_out, nullptr, 0};
+  return bgmv_batch(&one, 1, num_tokens, h_in, layer_idx, scale, 1, dtype, stream);
+}
+
+int lorax_bgmv_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems, int64_t num_tokens,
+                     int32_t h_in, int64_t layer_idx, float scale, int32_t accumulate, int32_t dtype,
+                     void* stream) {
+  return bgmv_batch(problems, num_problems, num_tokens, h_in, layer_idx, scale, accumulate, dtype, stream);
 }
 
 int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,

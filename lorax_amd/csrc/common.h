@@ -122,7 +122,7 @@ __device__ __forceinline__ int transpose_reduce_index(int lane) {
   return idx;
 }
 
-// Token grouping for BGMV.  Tokens that share indices[] value share one adapter; the
+// Token grouping for BGMV.  Tokens that share an indices[] value share one adapter; the
 // tokens of one adapter are cut, in token order, into chunks of at most G and the
 // first token of each chunk ("leader") processes the whole chunk, so the adapter's
 // weights are fetched once per chunk instead of once per token.
@@ -130,44 +130,63 @@ __device__ __forceinline__ int transpose_reduce_index(int lane) {
 // Called by every wave of the workgroup of token b with identical arguments; all
 // results are wave-uniform.  Returns the number of tokens in b's chunk (>= 1) if b
 // leads a chunk, with toks[0] = b and toks[1..] the followers in ascending order;
-// returns 0 if b is a follower (the workgroup has nothing to do).
+// returns 0 if b is a follower or has no adapter (the workgroup has nothing to do).
+// idx receives indices[b].
+//
+// The scan reads the index array in batches of kScanBlocks * 64 entries whose loads are
+// all issued before the first one is consumed, so a batch costs one memory round trip.
+constexpr int kScanBlocks = 8;
+
 template <int G>
 __device__ __forceinline__ int group_tokens(const int64_t* __restrict__ indices, int num_tokens,
-                                            int b, int64_t idx, int (&toks)[G]) {
+                                            int b, int64_t& idx, int (&toks)[G]) {
   const int lane = lane_id();
-  toks[0] = b;
 #pragma unroll
-  for (int g = 1; g < G; ++g) toks[g] = b;
-  if (G == 1) return 1;
-
-  // Rank of b among the tokens of its adapter = matches strictly before b.
-  int before = 0;
+  for (int g = 0; g < G; ++g) toks[g] = b;
   const int b_blk = b & ~(kWave - 1);
-  for (int t0 = 0; t0 < b_blk; t0 += kWave) {
-    const bool same = indices[t0 + lane] == idx;  // t0 + lane < b_blk <= num_tokens
-    before += __popcll(__ballot(same));
-  }
+  int before = 0;
   int n = 1;
-  for (int t0 = b_blk; t0 < num_tokens; t0 += kWave) {
-    const int t = t0 + lane;
-    const bool same = (t < num_tokens) && (indices[t] == idx);
-    uint64_t mask = __ballot(same);
-    if (t0 == b_blk) {
-      const uint64_t below = (1ull << (b - b_blk)) - 1ull;
-      before += __popcll(mask & below);
-      if ((before % G) != 0) return 0;
-      mask &= ~(below | (1ull << (b - b_blk)));
-    }
-    while (mask != 0 && n < G) {
-      const int pos = __ffsll(static_cast<unsigned long long>(mask)) - 1;
-      mask &= mask - 1;
+  bool first_batch = true;
+  for (int base = 0; base < num_tokens; base += kWave * kScanBlocks) {
+    int64_t vals[kScanBlocks];
 #pragma unroll
-      for (int g = 1; g < G; ++g) {
-        if (g == n) toks[g] = t0 + pos;
-      }
-      ++n;
+    for (int c = 0; c < kScanBlocks; ++c) {
+      const int t = base + c * kWave + lane;
+      vals[c] = t < num_tokens ? indices[t] : static_cast<int64_t>(-1);
     }
-    if (n == G) break;
+    if (first_batch) {
+      idx = indices[b];
+      if (idx < 0) return 0;
+      if (G == 1) return 1;
+      first_batch = false;
+    }
+#pragma unroll
+    for (int c = 0; c < kScanBlocks; ++c) {
+      const int t0 = base + c * kWave;
+      if (t0 < num_tokens) {
+        uint64_t mask = __ballot(vals[c] == idx);
+        if (t0 < b_blk) {
+          before += __popcll(mask);
+        } else {
+          if (t0 == b_blk) {
+            const uint64_t below = (1ull << (b - b_blk)) - 1ull;
+            before += __popcll(mask & below);
+            if ((before % G) != 0) return 0;
+            mask &= ~(below | (1ull << (b - b_blk)));
+          }
+          while (mask != 0 && n < G) {
+            const int pos = __ffsll(static_cast<unsigned long long>(mask)) - 1;
+            mask &= mask - 1;
+#pragma unroll
+            for (int g = 1; g < G; ++g) {
+              if (g == n) toks[g] = t0 + pos;
+            }
+            ++n;
+          }
+          if (n == G) return n;
+        }
+      }
+    }
   }
   return n;
 }

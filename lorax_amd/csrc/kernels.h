@@ -9,18 +9,40 @@
 
 namespace lorax {
 
-struct BgmvArgs {
+// One BGMV problem of a batched launch: its own output, input, pointer table and routing.
+// `width` is the problem's wide dimension (h_out of an expand); shrink problems of one
+// launch share h_in and rank, expand problems share the rank.
+struct BgmvProblem {
   void* y;
   const void* x;
   const int64_t* w_ptrs;
   const int64_t* indices;
-  int64_t num_tokens;
-  int h_in;
-  int h_out;
   int64_t y_offset;
   int64_t y_stride;
+  int width;
+  const int64_t* plan;  // optional routing plan: num_groups records of kPlanRecordWords int64
+  int num_groups;
+};
+
+constexpr int kMaxBgmvProblems = 4;
+constexpr int kPlanRecordWords = 8;
+
+struct BgmvBatch {
+  BgmvProblem p[kMaxBgmvProblems];
+};
+
+struct BgmvArgs {
+  BgmvBatch batch;
+  int count;          // problems in the batch (grid z)
+  bool expand;        // bgmv_impl.cuh:204: h_in < h_out
+  int narrow;         // LoRA rank
+  int wide_max;       // shrink: h_in; expand: widest h_out of the batch
+  int64_t num_tokens;
+  int64_t grid_rows;  // workgroup rows: tokens when chunks are found by scanning, else plan records
+  int64_t work_rows;  // estimate of the rows that have work (sizes the rows-per-workgroup choice)
   int64_t layer_idx;
   float scale;
+  int accumulate;     // shrink only: 0 = overwrite y, 1 = add to y
   int dtype;
 };
 

@@ -5,26 +5,29 @@ Mirrors ``lorax_server/utils/layers.py:59-300``: ``LoraLinear.forward_layer_type
 gate/up outputs, one column slice per layer name, :217-255) and
 ``TensorParallelAdapterRowLinear`` (o_proj / down_proj, :270-289).
 
-Two deliberate differences from the reference:
+Deliberate differences from the reference:
   * its third branch, the per-adapter masked matmul loop (:169-211), is not part of this
     package: a batch the kernels cannot take raises instead of silently running dense
     PyTorch code;
   * a projection that owns only a column slice of the fused output is written in place
     through the kernels' column window instead of through a zero-filled staging tensor
     and a second pass (:109-112,166-167).  Every token belongs to at most one rank
-    group, so both orders round identically.
+    group, so both orders round identically;
+  * in decode, the projections of one layer that share an input (q/k/v, gate/up) go to the
+    GPU as ONE shrink launch and ONE expand launch per rank (``lorax_bgmv_multi``), and the
+    shrink overwrites v, so there is no zero-fill (:146).  A decode-size BGMV is shorter
+    than a kernel launch; the reference issues 3 launches per projection and rank.
 """
 
-from typing import List, Optional
+from collections import defaultdict
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 from torch import nn
 
+from lorax_amd import _native
 from lorax_amd.adapters import LORA, AdapterBatchData, BatchLoraWeights
 from lorax_amd.sgmv import (
-    add_lora_a_bgmv,
-    add_lora_b_bgmv,
-    add_lora_b_bgmv_slice,
     has_sgmv,
     lora_a_sgmv_cutlass,
     lora_b_sgmv_cutlass,
@@ -49,6 +52,79 @@ class LoraLinear(nn.Module):
         self.layer_id = layer_id
         self.process_group = process_group if process_group is not None else SingleProcessGroup()
 
+    def _lora_data(self, adapter_data: AdapterBatchData, layer_type: str) -> Optional[BatchLoraWeights]:
+        layer_data = adapter_data.data.get(layer_type)
+        data = layer_data.get(LORA) if layer_data is not None else None
+        if data is None:
+            return None  # no adapter in the batch targets this projection
+        if not has_sgmv():
+            raise RuntimeError("LoRA kernels unavailable: liblorax_hip.so is not loaded or DISABLE_SGMV is set")
+        if not data.can_vectorize(self.process_group):
+            raise RuntimeError(
+                f"layer type {layer_type!r}: ranks {sorted(data.rank_data)} are outside what the LoRA kernels "
+                "cover (rank / world_size <= 128, not lm_head)"
+            )
+        return data
+
+    def forward_layer_types(
+        self,
+        result: torch.Tensor,
+        input: torch.Tensor,
+        adapter_data: AdapterBatchData,
+        slices: Sequence[Tuple[str, int, int]],
+    ) -> torch.Tensor:
+        """Adds the LoRA deltas of several projections that share `input`; projection `name` owns the
+        columns [start, end) of `result`."""
+        tensor_parallel = self.process_group.size() > 1
+        decode_jobs = defaultdict(list)  # rank -> [(rank_segments, start, width)]
+        for name, start, end in slices:
+            data = self._lora_data(adapter_data, name)
+            if data is None:
+                continue
+            sliced = end - start != result.shape[1]
+            for r, rs in data.rank_data.items():
+                if rs.lora_a_ptr is None or rs.lora_b_ptr is None:
+                    continue
+                if not data.use_sgmv:
+                    decode_jobs[r].append((rs, start, end - start))
+                    continue
+                v = lora_a_sgmv_cutlass(
+                    input, rs.tmp_shrink, rs.lora_a_ptr, rs.segment_starts, rs.segment_ends, self.layer_id, r
+                )
+                if tensor_parallel:
+                    v = self.collect_lora_a(v)
+                if sliced:
+                    lora_b_sgmv_cutlass_slice(
+                        result, v, rs.tmp_expand, rs.lora_b_ptr, rs.segment_starts, rs.segment_ends,
+                        self.layer_id, start, end - start,
+                    )
+                else:
+                    lora_b_sgmv_cutlass(
+                        result, v, rs.tmp_expand, rs.lora_b_ptr, rs.segment_starts, rs.segment_ends, self.layer_id
+                    )
+
+        step = _native.MAX_BGMV_PROBLEMS
+        for r, jobs in decode_jobs.items():
+            for i in range(0, len(jobs), step):
+                chunk = jobs[i : i + step]
+                # v needs no zero-fill: the shrink overwrites the rows of routed tokens and the
+                # expand reads no others
+                vs = torch.empty((len(chunk), input.size(0), r), dtype=input.dtype, device=input.device).unbind(0)
+                plans = [rs.plan for rs, _, _ in chunk]
+                if any(p is None for p in plans):
+                    plans = None  # tables not built by BatchLoraWeights.load: the kernels group tokens themselves
+                _native.bgmv_multi(
+                    [(v, input, rs.lora_a_ptr, rs.indices, 0, None) for v, (rs, _, _) in zip(vs, chunk)],
+                    self.layer_id, 1.0, accumulate=False, plans=plans,
+                )
+                if tensor_parallel:
+                    vs = [self.collect_lora_a(v) for v in vs]
+                _native.bgmv_multi(
+                    [(result, v, rs.lora_b_ptr, rs.indices, start, width) for v, (rs, start, width) in zip(vs, chunk)],
+                    self.layer_id, 1.0, accumulate=True, plans=plans,
+                )
+        return result
+
     def forward_layer_type(
         self,
         result: torch.Tensor,
@@ -58,70 +134,8 @@ class LoraLinear(nn.Module):
         start_idx: int,
         end_idx: int,
     ) -> torch.Tensor:
-        layer_data = adapter_data.data.get(layer_type)
-        data: Optional[BatchLoraWeights] = layer_data.get(LORA) if layer_data is not None else None
-        if data is None:
-            return result  # no adapter in the batch targets this projection
-        if not has_sgmv():
-            raise RuntimeError("LoRA kernels unavailable: liblorax_hip.so is not loaded or DISABLE_SGMV is set")
-        if not data.can_vectorize(self.process_group):
-            raise RuntimeError(
-                f"layer type {layer_type!r}: ranks {sorted(data.rank_data)} are outside what the LoRA kernels "
-                "cover (rank / world_size <= 128, not lm_head)"
-            )
-
-        sliced = end_idx - start_idx != result.shape[1]
-        tensor_parallel = self.process_group.size() > 1
-        for r, rank_segments in data.rank_data.items():
-            a_ptr, b_ptr = rank_segments.lora_a_ptr, rank_segments.lora_b_ptr
-            if a_ptr is None or b_ptr is None:
-                continue
-            if data.use_sgmv:
-                v = lora_a_sgmv_cutlass(
-                    input,
-                    rank_segments.tmp_shrink,
-                    a_ptr,
-                    rank_segments.segment_starts,
-                    rank_segments.segment_ends,
-                    self.layer_id,
-                    r,
-                )
-                if tensor_parallel:
-                    v = self.collect_lora_a(v)
-                if sliced:
-                    lora_b_sgmv_cutlass_slice(
-                        result,
-                        v,
-                        rank_segments.tmp_expand,
-                        b_ptr,
-                        rank_segments.segment_starts,
-                        rank_segments.segment_ends,
-                        self.layer_id,
-                        start_idx,
-                        end_idx - start_idx,
-                    )
-                else:
-                    lora_b_sgmv_cutlass(
-                        result,
-                        v,
-                        rank_segments.tmp_expand,
-                        b_ptr,
-                        rank_segments.segment_starts,
-                        rank_segments.segment_ends,
-                        self.layer_id,
-                    )
-            else:
-                v = torch.zeros((input.size(0), r), dtype=input.dtype, device=input.device)
-                add_lora_a_bgmv(v, input, a_ptr, rank_segments.indices, self.layer_id)
-                if tensor_parallel:
-                    v = self.collect_lora_a(v)
-                if sliced:
-                    add_lora_b_bgmv_slice(
-                        result, v, b_ptr, rank_segments.indices, self.layer_id, start_idx, end_idx - start_idx
-                    )
-                else:
-                    add_lora_b_bgmv(result, v, b_ptr, rank_segments.indices, self.layer_id)
-        return result
+        """One projection, with the reference's signature (utils/layers.py:66-74)."""
+        return self.forward_layer_types(result, input, adapter_data, [(layer_type, start_idx, end_idx)])
 
     def collect_lora_a(self, a_out: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError("tensor-parallel exchange of the shrink output is outside this package")
@@ -147,6 +161,7 @@ class TensorParallelMultiAdapterLinear(LoraLinear):
             input = input.reshape(-1, input.shape[-1])
             result = result.reshape(-1, result.shape[-1])
         world = self.process_group.size()
+        slices = []
         offset = 0
         for i, name in enumerate(self.layer_names):
             start = offset // world
@@ -155,7 +170,8 @@ class TensorParallelMultiAdapterLinear(LoraLinear):
                 end = offset // world
             else:
                 end = result.shape[1]
-            result = self.forward_layer_type(result, input, adapter_data, name, start, end)
+            slices.append((name, start, end))
+        result = self.forward_layer_types(result, input, adapter_data, slices)
         return result.reshape(out_shape)
 
 

@@ -190,3 +190,47 @@ def test_bgmv_errors_raise_runtime_error():
     sgmv.add_lora_a_bgmv(v, x, ptr, idx, 0)
     assert torch.all(v == 1)
     assert _native.available()
+
+
+@pytest.mark.parametrize("r", [8, 64])
+def test_bgmv_multi_matches_separate_launches(r):
+    """One batched launch for q/k/v (shared input, different widths, different routing per projection)
+    against the oracle; the overwrite mode of the shrink must not depend on what v held before."""
+    from lorax_amd import _native
+
+    dtype, T, h_in, n = torch.bfloat16, 100, 4096, 11
+    sizes = [4096, 1024, 1024]
+    gen = torch.Generator().manual_seed(21 + r)
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    y0 = randn((T, sum(sizes)), 0.5, gen, dtype, DEV)
+    y = y0.clone()
+    y_ref = y0.cpu().clone()
+    shrink, expand, vs, keep_alive = [], [], [], []
+    off = 0
+    for h_out in sizes:
+        wa_t = _stacks(n, 2, r, h_in, gen, dtype)
+        wb_t = _stacks(n, 2, h_out, r, gen, dtype)
+        keep_alive.append((wa_t, wb_t))  # the pointer tables hold raw addresses only
+        idx = _indices(T, n, gen, drop=0.15)  # routing differs between the projections
+        v = torch.full((T, r), float("nan"), dtype=dtype, device=DEV)
+        vs.append((v, idx))
+        shrink.append((v, x, ptr_table(wa_t, DEV), idx.to(DEV), 0, None))
+        expand.append((y, v, ptr_table(wb_t, DEV), idx.to(DEV), off, h_out))
+        v_ref = torch.zeros((T, r), dtype=dtype)
+        O.bgmv_ref(v_ref, x.cpu(), [w.cpu() for w in wa_t], idx.tolist(), 1)
+        part = y_ref[:, off:off + h_out].clone()
+        O.bgmv_ref(part, v_ref, [w.cpu() for w in wb_t], idx.tolist(), 1)
+        y_ref[:, off:off + h_out] = part
+        off += h_out
+    _native.bgmv_multi(shrink, 1, 1.0, accumulate=False)
+    _native.bgmv_multi(expand, 1, 1.0, accumulate=True)
+    torch.cuda.synchronize()
+    assert_close(y, y_ref, "fused q/k/v")
+    for v, idx in vs:
+        routed = idx >= 0
+        assert torch.isfinite(v.cpu()[routed].float()).all()
+        assert torch.isnan(v.cpu()[~routed].float()).all()  # rows without adapter are not written
+    with pytest.raises(RuntimeError, match="share direction and rank"):
+        _native.bgmv_multi([shrink[0], (torch.zeros((T, r + 8), dtype=dtype, device=DEV),) + shrink[1][1:]], 1)
+    with pytest.raises(RuntimeError, match="between 1 and 4"):
+        _native.bgmv_multi(shrink + shrink, 1)

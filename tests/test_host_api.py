@@ -241,3 +241,39 @@ def test_segmented_matmul():
     assert torch.allclose(y[0:2], x[0:2] @ w[0].t() + b[0])
     assert torch.allclose(y[3:6], x[3:6] @ w[1].t())
     assert torch.count_nonzero(y[2]) == 0
+
+
+def test_bgmv_plan_covers_every_routed_token_once():
+    from lorax_amd.adapters import BGMV_PLAN_GROUP, build_bgmv_plan
+
+    g = torch.Generator().manual_seed(3)
+    slots = torch.randint(-1, 7, (203,), generator=g).tolist()
+    a_addrs = [1000 + 16 * s for s in range(7)]
+    b_addrs = [9000 + 16 * s for s in range(7)]
+    records = build_bgmv_plan(slots, a_addrs, b_addrs)
+    seen = []
+    for rec in records:
+        n, toks, a, b, pad = rec[0], rec[1:5], rec[5], rec[6], rec[7]
+        assert 1 <= n <= BGMV_PLAN_GROUP and pad == 0 and len(rec) == 8
+        s = slots[toks[0]]
+        assert s >= 0 and (a, b) == (a_addrs[s], b_addrs[s])
+        assert all(slots[t] == s for t in toks[:n])
+        assert toks[:n] == sorted(toks[:n]) and all(t == toks[0] for t in toks[n:])
+        seen.extend(toks[:n])
+    assert sorted(seen) == [t for t, s in enumerate(slots) if s >= 0]
+    assert build_bgmv_plan([-1, -1], a_addrs, b_addrs) == []
+
+
+@pytest.mark.parametrize("case", _golden("lora_batch")["decode"])
+def test_decode_rank_groups_carry_a_plan(case):
+    layer = _layer(case["lora_ranks"])
+    meta = _meta(case["adapter_indices"])
+    data = layer.get_data(meta, LM_HEAD, prefill=False, prefill_head_indices=None).get(LORA)
+    for r, rd in data.rank_data.items():
+        idx = rd.indices.tolist()
+        assert rd.plan.dtype == torch.int64 and rd.plan.shape[1] == 8
+        covered = sorted(t for rec in rd.plan.tolist() for t in rec[1:1 + rec[0]])
+        assert covered == [t for t, s in enumerate(idx) if s >= 0]
+        for rec in rd.plan.tolist():
+            s = idx[rec[1]]
+            assert rec[5] == rd.lora_a_ptr[s].item() and rec[6] == rd.lora_b_ptr[s].item()
