@@ -41,6 +41,9 @@ def parse_args():
     p.add_argument("--pattern", choices=["fused", "reference"], default="fused",
                    help="launch sequence: the one lorax_amd.layers issues, or the reference caller's")
     p.add_argument("--no-plan", action="store_true", help="fused pattern without the host-built routing plan")
+    p.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                   help="also run a plain device copy of MIB MiB (3 times) so that a counter run holds a kernel of "
+                        "known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     p.add_argument("--eager", action="store_true", help="launch every step eagerly instead of replaying a graph")
     return p.parse_args()
 
@@ -291,6 +294,14 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     _native.init(device)
+
+    if args.calibrate_copy:
+        src = torch.ones(args.calibrate_copy << 20, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     w = build_workload(args.config, args.layers, device)
     L = w.num_layers

@@ -62,26 +62,39 @@ __device__ __forceinline__ void bgmv_shrink_body(typename D::E* __restrict__ Y,
 #pragma unroll
   for (int g = 0; g < NT; ++g) xrow[g] = X + static_cast<int64_t>(toks[g]) * h_in;
 
-#pragma unroll 2
-  for (int k = tid * 8; k < h_in; k += kBgmvThreads * 8) {
-    vec8 xv[NT];
-    vec8 wv[RS];
+  // Two hidden-dimension steps per trip: all loads of the trip are issued before the first
+  // one is consumed (the scheduling barrier keeps the compiler from sinking them to their
+  // uses), so a trip costs one memory round trip instead of one per row.
+  constexpr int kStep = kBgmvThreads * 8;
+  for (int k = tid * 8; k < h_in; k += 2 * kStep) {
+    vec8 xv[2][NT];
+    vec8 wv[2][RS];
+    const bool second = k + kStep < h_in;
 #pragma unroll
-    for (int g = 0; g < NT; ++g) xv[g] = load8<D>(xrow[g] + k);
+    for (int u = 0; u < 2; ++u) {
+      const int ku = k + u * kStep;
 #pragma unroll
-    for (int j = 0; j < RS; ++j) wv[j] = load8<D>(A + static_cast<int64_t>(j) * h_in + k);
-    float xf[NT][8];
+      for (int g = 0; g < NT; ++g) xv[u][g] = (u == 0 || second) ? load8<D>(xrow[g] + ku) : zero8<D>();
 #pragma unroll
-    for (int g = 0; g < NT; ++g)
+      for (int j = 0; j < RS; ++j)
+        wv[u][j] = (u == 0 || second) ? load8<D>(A + static_cast<int64_t>(j) * h_in + ku) : zero8<D>();
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) xf[g][e] = to_f32<D>(xv[g][e]);
+    for (int u = 0; u < 2; ++u) {
+      float xf[NT][8];
 #pragma unroll
-    for (int j = 0; j < RS; ++j) {
+      for (int g = 0; g < NT; ++g)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float w = to_f32<D>(wv[j][e]);
+        for (int e = 0; e < 8; ++e) xf[g][e] = to_f32<D>(xv[u][g][e]);
 #pragma unroll
-        for (int g = 0; g < NT; ++g) acc[j][g] = fmaf(w, xf[g][e], acc[j][g]);
+      for (int j = 0; j < RS; ++j) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float w = to_f32<D>(wv[u][j][e]);
+#pragma unroll
+          for (int g = 0; g < NT; ++g) acc[j][g] = fmaf(w, xf[g][e], acc[j][g]);
+        }
       }
     }
   }
@@ -108,16 +121,16 @@ __device__ __forceinline__ void bgmv_shrink_body(typename D::E* __restrict__ Y,
   }
 }
 
-// Resolves the token chunk of workgroup row blockIdx.y and the address of its adapter's stack.
+// Resolves the token chunk of workgroup row `row` and the address of its adapter's stack.
 // With a routing plan (built once per batch next to the index tables) this is one 64-byte
 // record: [ntok, tok0..tok3, address of the A stack, address of the B^T stack, reserved];
 // without one, the chunk is found by scanning indices[] (group_tokens).  Returns the number of
 // tokens, 0 if the workgroup has nothing to do.  Wave-uniform.
-__device__ __forceinline__ int resolve_chunk(const BgmvProblem& P, int num_tokens, bool expand,
+__device__ __forceinline__ int resolve_chunk(const BgmvProblem& P, int num_tokens, bool expand, int row,
                                              int (&toks)[kGroup], int64_t& stack_addr) {
   if (P.plan != nullptr) {
-    if (static_cast<int>(blockIdx.y) >= P.num_groups) return 0;
-    const int64_t* rec = P.plan + static_cast<int64_t>(blockIdx.y) * kPlanRecordWords;
+    if (row >= P.num_groups) return 0;
+    const int64_t* rec = P.plan + static_cast<int64_t>(row) * kPlanRecordWords;
     const int n = static_cast<int>(rec[0]);
 #pragma unroll
     for (int g = 0; g < kGroup; ++g) toks[g] = static_cast<int>(rec[1 + g]);
@@ -125,7 +138,7 @@ __device__ __forceinline__ int resolve_chunk(const BgmvProblem& P, int num_token
     return n;
   }
   int64_t idx;
-  const int n = group_tokens<kGroup>(P.indices, num_tokens, blockIdx.y, idx, toks);
+  const int n = group_tokens<kGroup>(P.indices, num_tokens, row, idx, toks);
   if (n == 0) return 0;
   stack_addr = P.w_ptrs[idx];
   return n;
@@ -137,12 +150,13 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_shrink_kernel(
     int accumulate_into_y) {
   __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<RS * kGroup>::value];
   using E = typename D::E;
-  const BgmvProblem& P = batch.p[blockIdx.z];
+  const VirtualBlock vb = xcd_virtual_block();
+  const BgmvProblem& P = batch.p[vb.z];
   int toks[kGroup];
   int64_t stack_addr;
-  const int n = resolve_chunk(P, num_tokens, false, toks, stack_addr);
+  const int n = resolve_chunk(P, num_tokens, false, vb.y, toks, stack_addr);
   if (n == 0) return;
-  const int row0 = blockIdx.x * RS;
+  const int row0 = vb.x * RS;
   const E* A = reinterpret_cast<const E*>(stack_addr) + (layer_idx * r + row0) * static_cast<int64_t>(h_in);
   E* Y = static_cast<E*>(P.y);
   const E* X = static_cast<const E*>(P.x);
@@ -238,13 +252,14 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBat
                                                                    int num_tokens, int r,
                                                                    int64_t layer_idx, float scale) {
   using E = typename D::E;
-  const BgmvProblem& P = batch.p[blockIdx.z];
+  const VirtualBlock vb = xcd_virtual_block();
+  const BgmvProblem& P = batch.p[vb.z];
   const int h_out = P.width;
-  const int col0 = blockIdx.x * (kBgmvThreads / CP) * U;
+  const int col0 = vb.x * (kBgmvThreads / CP) * U;
   if (col0 >= h_out) return;  // problems of one batch may differ in width
   int toks[kGroup];
   int64_t stack_addr;
-  const int n = resolve_chunk(P, num_tokens, true, toks, stack_addr);
+  const int n = resolve_chunk(P, num_tokens, true, vb.y, toks, stack_addr);
   if (n == 0) return;
   const E* B = reinterpret_cast<const E*>(stack_addr) + layer_idx * h_out * static_cast<int64_t>(r);
   E* Y = static_cast<E*>(P.y);

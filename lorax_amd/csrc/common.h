@@ -58,13 +58,26 @@ __device__ __forceinline__ void accumulate4(typename D::E* p, f32x4 delta) {
   *reinterpret_cast<vec4*>(p) = y;
 }
 
+// All tensors and weight stacks live in device (global) memory.  Weight addresses arrive as
+// integers, which the compiler can only treat as generic pointers (flat_load); the explicit
+// address space turns every 16-byte access into global_load/global_store_dwordx4.
+#define LORAX_GLOBAL __attribute__((address_space(1)))
+
 template <typename D>
 __device__ __forceinline__ typename D::vec8 load8(const typename D::E* p) {
-  return *reinterpret_cast<const typename D::vec8*>(p);
+  return *(const LORAX_GLOBAL typename D::vec8*)(p);
 }
 template <typename D>
 __device__ __forceinline__ void store8(typename D::E* p, typename D::vec8 v) {
-  *reinterpret_cast<typename D::vec8*>(p) = v;
+  *(LORAX_GLOBAL typename D::vec8*)(p) = v;
+}
+// v if keep, else zeros - a select on registers, for masking AFTER an unconditional load.
+template <typename D>
+__device__ __forceinline__ typename D::vec8 keep_if(bool keep, typename D::vec8 v) {
+  u32x4 bits = __builtin_bit_cast(u32x4, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) bits[i] = keep ? bits[i] : 0u;
+  return __builtin_bit_cast(typename D::vec8, bits);
 }
 template <typename D>
 __device__ __forceinline__ typename D::vec8 zero8() {
@@ -100,8 +113,13 @@ __device__ __forceinline__ void transpose_reduce(float (&vals)[N]) {
 #pragma unroll
     for (int i = 0; i < N / 2; ++i) {
       if (i < half) {
-        const float keep = upper ? vals[i + half] : vals[i];
-        const float send = upper ? vals[i] : vals[i + half];
+        float lo = vals[i];
+        float hi = vals[i + half];
+        // Opaque to the optimiser: without this it rewrites "upper ? vals[i + half] : vals[i]"
+        // into a load with a lane-dependent index, which costs an N-way select chain per access.
+        asm volatile("" : "+v"(lo), "+v"(hi));
+        const float keep = upper ? hi : lo;
+        const float send = upper ? lo : hi;
         vals[i] = keep + __shfl_xor(send, m, kWave);
       }
     }
@@ -120,6 +138,32 @@ __device__ __forceinline__ int transpose_reduce_index(int lane) {
     if (lane & m) idx += n >> 1;
   }
   return idx;
+}
+
+// XCD-aware workgroup numbering.  The 8 XCDs of an MI355X each have their own L2 and receive
+// workgroups round-robin by linear workgroup id, so neighbours in the grid never share an L2.
+// This maps the hardware id to a virtual (x, y, z) in which consecutive virtual ids - x fastest,
+// then z, then y - run on ONE XCD: the workgroups that read the same activation rows (all row or
+// column slices and all batched problems of one token chunk) then hit the same L2 instead of
+// fetching those rows once per XCD.
+constexpr unsigned kXcds = 8;
+
+struct VirtualBlock {
+  int x, y, z;
+};
+
+__device__ __forceinline__ VirtualBlock xcd_virtual_block() {
+  const unsigned gx = gridDim.x, gy = gridDim.y, gz = gridDim.z;
+  const unsigned n = gx * gy * gz;
+  const unsigned lin = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+  const unsigned per = n / kXcds, rem = n % kXcds;  // XCD k runs per + (k < rem) workgroups
+  const unsigned xcd = lin % kXcds, slot = lin / kXcds;
+  const unsigned v = xcd * per + (xcd < rem ? xcd : rem) + slot;
+  VirtualBlock b;
+  b.x = static_cast<int>(v % gx);
+  b.z = static_cast<int>((v / gx) % gz);
+  b.y = static_cast<int>(v / (gx * gz));
+  return b;
 }
 
 // Token grouping for BGMV.  Tokens that share an indices[] value share one adapter; the

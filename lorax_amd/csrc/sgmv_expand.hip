@@ -26,6 +26,7 @@ constexpr int kExpandBlocksPerWave = 4;  // 16-row blocks per wave and tile
 constexpr int kExpandRows = 16 * kExpandWaves * kExpandBlocksPerWave;  // rows per tile
 constexpr int kExpandShortRows = 4;      // row tiles up to this height use the vector path
 constexpr int kPanelPitch = kExpandCols + 4;  // LDS row pitch in elements
+constexpr int kExpandStages = 3;              // register stages of the row-block pipeline
 
 // Output column (0..63) that row `a` of the first MFMA operand of accumulator j
 // stands for.  Chosen so that lane group g = a / 4 ends up with columns
@@ -132,22 +133,31 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
     const int nmb = (nrows + 15) / 16;
     const bool col_ok0 = n0 + g * 8 < h_out;
     const bool col_ok1 = n0 + 32 + g * 8 < h_out;
-    auto load_block = [&](int mb, vec8(&vf)[KS], vec8& y0, vec8& y1) {
-      const int row = rt.row0 + mb * 16 + c;
-      const bool ok = row < rt.row_end;
+    // Loads are unconditional: rows past the tile are clamped to its last row and columns past
+    // h_out to the panel's first vector (both valid memory); only the stores are predicated.
+    // v chunks beyond the rank are zeroed after the load.
+    const int coff0 = col_ok0 ? g * 8 : 0;
+    const int coff1 = col_ok1 ? 32 + g * 8 : 0;
+    bool k_ok[KS];
+    int k_off[KS];
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        vf[s] = zero8<D>();
-        if (ok && s * 32 + g * 8 < r) vf[s] = load8<D>(V + static_cast<int64_t>(row) * r + s * 32 + g * 8);
-      }
-      const E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0 + g * 8;
-      y0 = zero8<D>();
-      y1 = zero8<D>();
-      if (ok && col_ok0) y0 = load8<D>(yp);
-      if (ok && col_ok1) y1 = load8<D>(yp + 32);
+    for (int s = 0; s < KS; ++s) {
+      k_ok[s] = s * 32 + g * 8 < r;
+      k_off[s] = k_ok[s] ? s * 32 + g * 8 : 0;
+    }
+    auto load_block = [&](int mb, vec8(&vf)[KS], vec8& y0, vec8& y1) {
+      const int row = min(rt.row0 + mb * 16 + c, rt.row_end - 1);
+      const E* vp = V + static_cast<int64_t>(row) * r;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) vf[s] = load8<D>(vp + k_off[s]);
+      const E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0;
+      y0 = load8<D>(yp + coff0);
+      y1 = load8<D>(yp + coff1);
     };
-    auto finish_block = [&](int mb, const vec8(&vf)[KS], vec8 y0, vec8 y1) {
+    auto finish_block = [&](bool live, int mb, vec8(&vf)[KS], vec8 y0, vec8 y1) {
       f32x4 acc[4];
+#pragma unroll
+      for (int s = 0; s < KS; ++s) vf[s] = keep_if<D>(k_ok[s], vf[s]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -155,8 +165,8 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
         for (int s = 0; s < KS; ++s) acc[j] = D::mfma16(bf[j][s], vf[s], acc[j]);
       }
       const int row = rt.row0 + mb * 16 + c;
-      const bool ok = row < rt.row_end;
-      E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0 + g * 8;
+      const bool ok = live && row < rt.row_end;
+      E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         y0[i] = accumulate<D>(y0[i], acc[0][i]);
@@ -164,24 +174,29 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
         y1[i] = accumulate<D>(y1[i], acc[2][i]);
         y1[4 + i] = accumulate<D>(y1[4 + i], acc[3][i]);
       }
-      if (ok && col_ok0) store8<D>(yp, y0);
-      if (ok && col_ok1) store8<D>(yp + 32, y1);
+      if (ok && col_ok0) store8<D>(yp + g * 8, y0);
+      if (ok && col_ok1) store8<D>(yp + 32 + g * 8, y1);
     };
 
-    int mb = wave;
-    if (mb < nmb) {
-      vec8 va[KS], vb[KS], ya0, ya1, yb0, yb1;
-      load_block(mb, va, ya0, ya1);
-      while (true) {
-        const int mb2 = mb + kExpandWaves;
-        if (mb2 < nmb) load_block(mb2, vb, yb0, yb1);
-        finish_block(mb, va, ya0, ya1);
-        if (mb2 >= nmb) break;
-        const int mb3 = mb2 + kExpandWaves;
-        if (mb3 < nmb) load_block(mb3, va, ya0, ya1);
-        finish_block(mb2, vb, yb0, yb1);
-        if (mb3 >= nmb) break;
-        mb = mb3;
+    // This wave's 16-row blocks are wave, wave + 4, ... below nmb.  They run through a ring of
+    // kExpandStages register stages (static indices, unrolled): the y and v loads of the next
+    // kExpandStages-1 blocks are in flight while one block is multiplied and stored.  Surplus
+    // trips of the last round re-load the last block and store nothing.
+    if (wave < nmb) {
+      const int n = (nmb - wave + kExpandWaves - 1) / kExpandWaves;
+      auto block_of = [&](int i) { return wave + min(i, n - 1) * kExpandWaves; };
+      vec8 vr[kExpandStages][KS], y0r[kExpandStages], y1r[kExpandStages];
+#pragma unroll
+      for (int s = 0; s < kExpandStages - 1; ++s) load_block(block_of(s), vr[s], y0r[s], y1r[s]);
+      for (int i = 0; i < n; i += kExpandStages) {
+#pragma unroll
+        for (int s = 0; s < kExpandStages; ++s) {
+          constexpr int kAhead = kExpandStages - 1;
+          load_block(block_of(i + s + kAhead), vr[(s + kAhead) % kExpandStages], y0r[(s + kAhead) % kExpandStages],
+                     y1r[(s + kAhead) % kExpandStages]);
+          __builtin_amdgcn_sched_barrier(0);
+          finish_block(i + s < n, block_of(i + s), vr[s], y0r[s], y1r[s]);
+        }
       }
     }
   }

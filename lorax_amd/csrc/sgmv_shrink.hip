@@ -31,6 +31,8 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
   constexpr int R = NB * 16;
   constexpr int ROWS = MB * 16;
   constexpr int THREADS = WAVES * kWave;
+  // register stages of the K pipeline: as many as fit next to the accumulators
+  constexpr int STAGES = (MB + NB) * 4 * 4 + MB * NB * 4 <= 200 ? 4 : ((MB + NB) * 4 * 3 + MB * NB * 4 <= 232 ? 3 : 2);
   __shared__ f32x4 red[WAVES][NB][kWave];
   __shared__ uint32_t arrival;
 
@@ -55,13 +57,14 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
     const int nmb = (rt.row_end - rt.row0 + 15) / 16;
     const E* A = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * R * static_cast<int64_t>(h_in);
 
+    // Operand addresses.  Rows past the end of the tile are clamped to its last row: they load
+    // valid memory, produce output rows nobody stores, and keep the loop free of conditional
+    // loads (a load into a register that was just zeroed makes the compiler wait for it).
     const E* xp[MB];
-    bool xok[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      const int row = rt.row0 + mb * 16 + c;
-      xok[mb] = row < rt.row_end;
-      xp[mb] = X + static_cast<int64_t>(xok[mb] ? row : rt.row0) * h_in + g * 8;
+      const int row = min(rt.row0 + mb * 16 + c, rt.row_end - 1);
+      xp[mb] = X + static_cast<int64_t>(row) * h_in + g * 8;
     }
     const E* ap = A + static_cast<int64_t>(c) * h_in + g * 8;
 
@@ -73,43 +76,54 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
 
     auto load_step = [&](int ks, vec8(&xf)[MB], vec8(&wf)[NB]) {
       const int k = ks * 32;
-      const bool kok = k + g * 8 < h_in;
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        xf[mb] = zero8<D>();
-        if (mb < nmb && kok && xok[mb]) xf[mb] = load8<D>(xp[mb] + k);
-      }
+      for (int mb = 0; mb < MB; ++mb) xf[mb] = load8<D>(xp[mb] + k);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        wf[nb] = zero8<D>();
-        if (kok) wf[nb] = load8<D>(ap + static_cast<int64_t>(nb) * 16 * h_in + k);
-      }
+      for (int nb = 0; nb < NB; ++nb) wf[nb] = load8<D>(ap + static_cast<int64_t>(nb) * 16 * h_in + k);
     };
-    auto mma_step = [&](const vec8(&xf)[MB], const vec8(&wf)[NB]) {
+    auto mma_step = [&](bool live, vec8(&xf)[MB], const vec8(&wf)[NB]) {
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        if (mb < nmb) {
+        const vec8 xm = keep_if<D>(live, xf[mb]);
 #pragma unroll
-          for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = D::mfma16(wf[nb], xf[mb], acc[mb][nb]);
-        }
+        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = D::mfma16(wf[nb], xm, acc[mb][nb]);
       }
     };
 
-    // Two-stage register pipeline over this wave's K steps.
-    int ks = ks0 + wave;
-    if (ks < ks1) {
-      vec8 xa[MB], wa[NB], xb[MB], wb[NB];
-      load_step(ks, xa, wa);
-      while (true) {
-        const int ks2 = ks + WAVES;
-        if (ks2 < ks1) load_step(ks2, xb, wb);
-        mma_step(xa, wa);
-        if (ks2 >= ks1) break;
-        const int ks3 = ks2 + WAVES;
-        if (ks3 < ks1) load_step(ks3, xa, wa);
-        mma_step(xb, wb);
-        if (ks3 >= ks1) break;
-        ks = ks3;
+    // This wave's K steps are ks0 + wave, + WAVES, ... below `last` (whole steps only).  They run
+    // through a ring of STAGES register stages with STAGES-1 steps of loads in flight while one
+    // step multiplies.  The ring is unrolled, so stage indices are static; the trip count is
+    // rounded up to a multiple of STAGES, the surplus steps re-load the last step (clamped
+    // address) and multiply zeros.
+    const int last = min(ks1, h_in / 32);
+    const int first = ks0 + wave;
+    if (first < last) {
+      const int n = (last - first + WAVES - 1) / WAVES;
+      auto step_ks = [&](int i) { return first + min(i, n - 1) * WAVES; };
+      vec8 xr[STAGES][MB], wr[STAGES][NB];
+#pragma unroll
+      for (int s = 0; s < STAGES - 1; ++s) load_step(step_ks(s), xr[s], wr[s]);
+      for (int i = 0; i < n; i += STAGES) {
+#pragma unroll
+        for (int s = 0; s < STAGES; ++s) {
+          load_step(step_ks(i + s + STAGES - 1), xr[(s + STAGES - 1) % STAGES], wr[(s + STAGES - 1) % STAGES]);
+          __builtin_amdgcn_sched_barrier(0);
+          mma_step(i + s < n, xr[s], wr[s]);
+        }
+      }
+    }
+    // A hidden size that is not a multiple of 32 leaves one partial step: the lanes whose 8 k
+    // lie beyond h_in contribute zeros.
+    if ((h_in & 31) != 0) {
+      const int kt = h_in / 32;
+      if (kt >= ks0 && kt < ks1 && (kt - ks0) % WAVES == wave) {
+        const bool kok = kt * 32 + g * 8 < h_in;
+        const int k = kok ? kt * 32 : 0;
+        vec8 xt[MB], wt[NB];
+        load_step(k / 32, xt, wt);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) wt[nb] = keep_if<D>(kok, wt[nb]);
+        mma_step(kok, xt, wt);
       }
     }
 
@@ -260,17 +274,18 @@ static hipError_t launch_rh_nb(const SgmvArgs& a, hipStream_t stream) {
   if (mb != 1 && mb != 2 && mb != 4) mb = 1;
   if (NB > 4 && mb > 2) mb = 2;
 
-  // Split K across workgroups until there are about four workgroups per CU, as long
-  // as every wave keeps at least two K steps and the partial sums fit the workspace.
+  // Splitting K across workgroups costs a device-scope fence per workgroup, which is only worth
+  // paying when the row tiles alone cannot occupy the 256 CUs.
   const int64_t tiles = (a.num_tokens + mb * 16 - 1) / (mb * 16) + a.num_segments;
   const int ksteps = (a.d_in + 31) / 32;
   int ksplit = 1;
   if (tuning().shrink_ksplit > 0) {
     ksplit = tuning().shrink_ksplit;
-  } else {
-    const int64_t want = (1024 + tiles - 1) / tiles;
-    const int kmax = ksteps / 8 > 0 ? ksteps / 8 : 1;
+  } else if (tiles < 192) {
+    const int64_t want = (384 + tiles - 1) / tiles;
+    const int kmax = ksteps / 16 > 0 ? ksteps / 16 : 1;
     ksplit = static_cast<int>(want < kmax ? want : kmax);
+    if (ksplit > 8) ksplit = 8;
   }
   if (ksplit > ksteps) ksplit = ksteps;
   if (ksplit < 1) ksplit = 1;
