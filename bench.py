@@ -44,6 +44,8 @@ def parse_args():
     p.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                    help="also run a plain device copy of MIB MiB (3 times) so that a counter run holds a kernel of "
                         "known traffic to scale FETCH_SIZE / WRITE_SIZE by")
+    p.add_argument("--two-launch", action="store_true",
+                   help="fused pattern without the single-launch shrink+expand kernel for ranks 8 and 16")
     p.add_argument("--eager", action="store_true", help="launch every step eagerly instead of replaying a graph")
     return p.parse_args()
 
@@ -68,13 +70,15 @@ class Plan:
     caller's sequence (utils/layers.py:114-164): zero-fill, shrink, expand for every projection and rank.
     """
 
-    def __init__(self, w, pattern="fused", use_plan=True):
+    def __init__(self, w, pattern="fused", use_plan=True, fuse_small_ranks=True):
         import torch
 
+        from lorax_amd import _native
         from lorax_amd.adapters import LORA
 
         self.w = w
         self.use_plan = use_plan
+        self.fuse_small_ranks = fuse_small_ranks
         self.batch = w.batch_data()
         self.calls = []  # (kind, fn(layer), algorithmic bytes, flops)
         T = w.num_tokens
@@ -97,9 +101,15 @@ class Plan:
                     self._add_bgmv_reference(x, y, off, size, group.h_in, r, rd)
                 else:
                     decode[r].append((rd, off, size))
-            for r, chunk_jobs in decode.items():
-                for i in range(0, len(chunk_jobs), 4):
-                    self._add_bgmv_fused(x, y, group.h_in, r, chunk_jobs[i:i + 4])
+            for r, rank_jobs in decode.items():
+                single = []
+                if self.use_plan and self.fuse_small_ranks:
+                    single = [j for j in rank_jobs if _native.bgmv_lora_fits(r, group.h_in, j[2])]
+                    rank_jobs = [j for j in rank_jobs if not any(j is s for s in single)]
+                for i in range(0, len(single), 4):
+                    self._add_bgmv_fused(x, y, group.h_in, r, single[i:i + 4], single_launch=True)
+                for i in range(0, len(rank_jobs), 4):
+                    self._add_bgmv_fused(x, y, group.h_in, r, rank_jobs[i:i + 4], single_launch=False)
 
     @staticmethod
     def _bgmv_counts(rd):
@@ -153,7 +163,7 @@ class Plan:
                            lambda layer: sgmv.add_lora_b_bgmv_slice(y, v, b_ptr, idx, layer, off, size),
                            rows * r * e + uniq * r * size * e + 2 * rows * size * e, 2 * rows * r * size))
 
-    def _add_bgmv_fused(self, x, y, h_in, r, jobs):
+    def _add_bgmv_fused(self, x, y, h_in, r, jobs, single_launch):
         import torch
 
         from lorax_amd import _native
@@ -169,6 +179,14 @@ class Plan:
         expand_bytes = sum(n * r * e + u * r * size * e + 2 * n * size * e
                            for (n, u), (_, _, size) in zip(counts, jobs))
         plans = [rd.plan for rd, _, _ in jobs] if self.use_plan else None
+        if single_launch:
+            lora_problems = [(y, x, rd.plan, off, size) for rd, off, size in jobs]
+            # v stays on chip: its write by the shrink and read by the expand are not memory traffic
+            v_bytes = sum(2 * n * r * e for n, _ in counts)
+            self.calls.append(("bgmv_lora", lambda layer: _native.bgmv_lora_multi(lora_problems, r, layer),
+                               shrink_bytes + expand_bytes - v_bytes,
+                               sum(2 * n * r * (h_in + size) for (n, _), (_, _, size) in zip(counts, jobs))))
+            return
         self.calls.append(("bgmv_shrink", lambda layer: _native.bgmv_multi(shrink_problems, layer, 1.0, False, plans),
                            shrink_bytes, sum(2 * n * r * h_in for n, _ in counts)))
         self.calls.append(("bgmv_expand", lambda layer: _native.bgmv_multi(expand_problems, layer, 1.0, True, plans),
@@ -305,7 +323,7 @@ def main():
 
     w = build_workload(args.config, args.layers, device)
     L = w.num_layers
-    plan = Plan(w, args.pattern, not args.no_plan)
+    plan = Plan(w, args.pattern, not args.no_plan, not args.two_launch)
     torch.cuda.synchronize()
 
     if args.eager:

@@ -112,6 +112,20 @@ int lorax_bgmv_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems,
                      void* stream);
 
 /*
+ * Shrink and expand of up to 4 projections in one launch: for every planned token chunk
+ *   y[t, y_offset : y_offset + h_out] += dtype(scale * dtype(x[t] @ A^T) @ B^T)
+ * with A and B^T taken from plan words [5] and [6].  No counterpart in the reference (it is the
+ * pair add_lora_a_bgmv + add_lora_b_bgmv of lorax_server/utils/layers.py:146-164 without the
+ * intermediate v tensor and the second launch).  Every problem needs a routing plan; the rank r
+ * must be 8 or 16, because each column slice of a projection recomputes the shrink and the
+ * adapter's A slab has to be small for that to pay.  The intermediate x @ A^T is rounded to
+ * dtype exactly as the two-call sequence rounds it when it stores v.
+ */
+int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems, int64_t num_tokens,
+                          int32_t h_in, int32_t r, int64_t layer_idx, float scale, int32_t dtype,
+                          void* stream);
+
+/*
  * SGMV shrink.  Replaces sgmv_shrink (punica_ops.cc:369-411,
  * sgmv_flashinfer/sgmv_all.cu:10-65) for a_layout = LORAX_A_RH and the shrink
  * direction of sgmv_cutlass (punica_ops.cc:338-367, sgmv/sgmv_cutlass.cuh:132-178)

@@ -53,6 +53,11 @@ _SIGNATURES = {
         [_c.POINTER(BgmvProblem), _c.c_int32, _c.c_int64, _c.c_int32, _c.c_int64, _c.c_float, _c.c_int32,
          _c.c_int32, _c.c_void_p],
     ),
+    "lorax_bgmv_lora_multi": (
+        _c.c_int,
+        [_c.POINTER(BgmvProblem), _c.c_int32, _c.c_int64, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float,
+         _c.c_int32, _c.c_void_p],
+    ),
     "lorax_sgmv_shrink": (
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
@@ -240,6 +245,48 @@ def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> N
     with torch.cuda.device(x0.device):
         rc = lib().lorax_bgmv_multi(arr, len(problems), x0.size(0), x0.size(1), int(layer_idx), float(scale),
                                     1 if accumulate else 0, _dtype_code(x0), _stream(x0))
+    if rc != 0:
+        _raise_last(rc)
+
+
+FUSED_BGMV_RANKS = (8, 16)
+
+
+def bgmv_lora_fits(rank: int, h_in: int, h_out: int) -> bool:
+    """True where the single-launch shrink+expand (lorax_bgmv_lora_multi) is the better choice: the adapter's
+    A slab is small (<= 128 KiB) and one workgroup covers all output columns of the projection (4096 at
+    rank 8, 2048 at rank 16), so no column slice has to repeat the shrink. Wider or deeper projections are
+    faster as a shrink launch plus an expand launch."""
+    if rank not in FUSED_BGMV_RANKS:
+        return False
+    return rank * h_in * 2 <= 128 * 1024 and h_out <= (256 // (rank // 8)) * 16
+
+
+def bgmv_lora_multi(problems, rank, layer_idx, scale=1.0) -> None:
+    """lorax_bgmv_lora_multi: `problems` is a list of up to 4 tuples (y, x, plan, y_offset, y_slice_size) that
+    share x.shape; y[:, window] += (x @ A^T) @ B^T per planned token chunk, rank 8 or 16."""
+    if not 1 <= len(problems) <= MAX_BGMV_PROBLEMS:
+        raise RuntimeError(f"between 1 and {MAX_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
+    arr = (BgmvProblem * len(problems))()
+    x0 = problems[0][1]
+    for i, (y, x, plan, y_offset, y_slice_size) in enumerate(problems):
+        _check_input(y, "y", 2)
+        _check_input(x, "x", 2)
+        _check_input(plan, "plan", 2)
+        _check_same(y, x, plan)
+        if x.shape != x0.shape or x.dtype != x0.dtype or x.device != x0.device:
+            raise RuntimeError("all problems of one launch must have inputs of one shape, dtype and device")
+        if y.size(0) != x.size(0):
+            raise RuntimeError(f"CHECK_EQ(y.size(0), x.size(0)) failed. {y.size(0)} vs {x.size(0)}")
+        if plan.dtype != torch.int64 or plan.size(1) != PLAN_RECORD_WORDS:
+            raise RuntimeError(f"plan must be an int64 [num_groups, {PLAN_RECORD_WORDS}] tensor on the device of x")
+        h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
+        plan_ptr = plan.data_ptr() if plan.size(0) > 0 else x.data_ptr()
+        arr[i] = BgmvProblem(y.data_ptr(), x.data_ptr(), None, None, int(y_offset), y.size(1), h_out, plan_ptr,
+                             plan.size(0))
+    with torch.cuda.device(x0.device):
+        rc = lib().lorax_bgmv_lora_multi(arr, len(problems), x0.size(0), x0.size(1), int(rank), int(layer_idx),
+                                         float(scale), _dtype_code(x0), _stream(x0))
     if rc != 0:
         _raise_last(rc)
 

@@ -41,30 +41,31 @@ def hipcc() -> str:
 
 def _compile(src: str, obj_dir: Path) -> Path:
     obj = obj_dir / (Path(src).stem + ".o")
-    cmd = [hipcc(), *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+    extra = os.environ.get("LORAX_EXTRA_HIPCC_FLAGS", "").split()  # e.g. -DLORAX_EXPAND_STAGES=4 for tuning builds
+    cmd = [hipcc(), *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{proc.stderr}")
     return obj
 
 
-def build(verbose: bool = True) -> Path:
+def build(verbose: bool = True, out: Path = LIB_PATH) -> Path:
     """Compiles every source and links the shared library. Always recompiles."""
     obj_dir = PKG_DIR / "build"
     obj_dir.mkdir(exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
         objs = list(pool.map(lambda s: _compile(s, obj_dir), SOURCES))
-    tmp = LIB_PATH.with_suffix(".so.tmp")
+    tmp = Path(str(out) + ".tmp")
     cmd = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stderr}")
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, out)
     if verbose:
-        print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
-    return LIB_PATH
+        print(f"built {out} ({out.stat().st_size} bytes)")
+    return out
 
 
 if __name__ == "__main__":
-    build()
+    build(out=Path(sys.argv[1]).resolve() if len(sys.argv) > 1 else LIB_PATH)
     sys.exit(0)

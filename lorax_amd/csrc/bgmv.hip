@@ -81,22 +81,11 @@ __device__ __forceinline__ void bgmv_shrink_body(typename D::E* __restrict__ Y,
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      float xf[NT][8];
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int g = 0; g < NT; ++g)
+      for (int j = 0; j < RS; ++j)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) xf[g][e] = to_f32<D>(xv[u][g][e]);
-#pragma unroll
-      for (int j = 0; j < RS; ++j) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float w = to_f32<D>(wv[u][j][e]);
-#pragma unroll
-          for (int g = 0; g < NT; ++g) acc[j][g] = fmaf(w, xf[g][e], acc[j][g]);
-        }
-      }
-    }
+        for (int g = 0; g < NT; ++g) acc[j][g] = dot8<D>(wv[u][j], xv[u][g], acc[j][g]);
   }
 
   // Wave reduction of the RS*NT sums, then across the four waves through LDS.
@@ -197,13 +186,11 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
   const int part = tid % CP;
   const bool has_k = part * 8 < r;
 
-  float vf[NT][8];
+  vec8 vv[NT];
 #pragma unroll
   for (int g = 0; g < NT; ++g) {
-    vec8 vv = zero8<D>();
-    if (has_k) vv = load8<D>(V + static_cast<int64_t>(toks[g]) * r + part * 8);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) vf[g][e] = to_f32<D>(vv[e]);
+    vv[g] = zero8<D>();
+    if (has_k) vv[g] = load8<D>(V + static_cast<int64_t>(toks[g]) * r + part * 8);
   }
 
   vec8 wv[U];
@@ -227,13 +214,7 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
   for (int u = 0; u < U; ++u) {
     float s[NT];
 #pragma unroll
-    for (int g = 0; g < NT; ++g) s[g] = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float w = to_f32<D>(wv[u][e]);
-#pragma unroll
-      for (int g = 0; g < NT; ++g) s[g] = fmaf(w, vf[g][e], s[g]);
-    }
+    for (int g = 0; g < NT; ++g) s[g] = dot8<D>(wv[u], vv[g], 0.f);
 #pragma unroll
     for (int m = CP / 2; m >= 1; m >>= 1)
 #pragma unroll
@@ -276,6 +257,187 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBat
       break;
     default:
       bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
+      break;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Shrink and expand of one projection in ONE launch, for ranks whose A slab is small enough
+// that every column slice can afford to recompute the shrink (rank 8 and 16): a workgroup
+// issues the loads of its slice of B^T and of the old y first (they do not depend on v), runs
+// the whole shrink of its token chunk (all R rows, full hidden dimension; the slab is shared
+// through L2 by the slices of the chunk, which the XCD-aware numbering puts on one XCD), rounds
+// v to the storage type exactly where the two-launch path would store it, and finishes with
+// the expand of its columns.  v never goes to memory and one launch boundary disappears.
+// ---------------------------------------------------------------------------------
+template <typename D, int R, int U, int NBLK, int NT>
+__device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
+                                               const typename D::E* __restrict__ X,
+                                               const typename D::E* __restrict__ A,
+                                               const typename D::E* __restrict__ B,
+                                               const int (&toks)[kGroup], int h_in, int h_out, int col0,
+                                               int col_end, int64_t y_offset, int64_t y_stride, float scale,
+                                               float* red, typename D::E* vsh) {
+  using vec8 = typename D::vec8;
+  using E = typename D::E;
+  constexpr int CP = R / 8;
+  constexpr int kCols = kBgmvThreads / CP;     // columns per step of the workgroup
+  constexpr int kBlock = kCols * U;            // columns per expand block
+  constexpr int kSteps = R <= 8 ? 2 : 1;       // hidden-dimension steps per trip (register budget)
+  const int tid = threadIdx.x;
+  const int part = tid % CP;
+
+  E* yrow[NT];
+#pragma unroll
+  for (int g = 0; g < NT; ++g) yrow[g] = Y + static_cast<int64_t>(toks[g]) * y_stride + y_offset;
+
+  // (1) every B^T vector of the workgroup's column range goes out before the shrink: they do
+  // not depend on v, and being cold they are the long pole of the expand.  Clamped, not predicated.
+  auto column = [&](int blk, int u) { return col0 + blk * kBlock + u * kCols + tid / CP; };
+  vec8 wv[NBLK][U];
+#pragma unroll
+  for (int blk = 0; blk < NBLK; ++blk)
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      wv[blk][u] = load8<D>(B + static_cast<int64_t>(min(column(blk, u), h_out - 1)) * R + part * 8);
+  // the old y of one block (warm: the base projection has just written it)
+  auto load_y = [&](int blk, E(&yv)[U][NT]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int cc = min(column(blk, u), h_out - 1);
+#pragma unroll
+      for (int g = 0; g < NT; ++g) yv[u][g] = yrow[g][cc];
+    }
+  };
+
+  // (2) shrink: all R rows of the slab against the chunk's tokens
+  float acc[R][NT];
+#pragma unroll
+  for (int j = 0; j < R; ++j)
+#pragma unroll
+    for (int g = 0; g < NT; ++g) acc[j][g] = 0.f;
+  const E* xrow[NT];
+#pragma unroll
+  for (int g = 0; g < NT; ++g) xrow[g] = X + static_cast<int64_t>(toks[g]) * h_in;
+  constexpr int kStep = kBgmvThreads * 8;
+  for (int k = tid * 8; k < h_in; k += kSteps * kStep) {
+    vec8 xv[kSteps][NT];
+    vec8 av[kSteps][R];
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+      // a step past the end re-reads the thread's first chunk and is masked to zero below
+      const bool live = k + u * kStep < h_in;
+      const int ku = live ? k + u * kStep : tid * 8;
+#pragma unroll
+      for (int g = 0; g < NT; ++g) xv[u][g] = keep_if<D>(live, load8<D>(xrow[g] + ku));
+#pragma unroll
+      for (int j = 0; j < R; ++j) av[u][j] = load8<D>(A + static_cast<int64_t>(j) * h_in + ku);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u)
+#pragma unroll
+      for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int g = 0; g < NT; ++g) acc[j][g] = dot8<D>(av[u][j], xv[u][g], acc[j][g]);
+  }
+
+  // (3) workgroup-wide sums -> v in LDS, rounded to the storage type
+  constexpr int NV = Pow2Ceil<R * NT>::value;
+  float vals[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) vals[i] = 0.f;
+#pragma unroll
+  for (int j = 0; j < R; ++j)
+#pragma unroll
+    for (int g = 0; g < NT; ++g) vals[g * R + j] = acc[j][g];
+  transpose_reduce<NV>(vals);
+  const int lane = lane_id();
+  const int wave = tid / kWave;
+  if ((lane & (kWave / NV - 1)) == 0) red[wave * NV + transpose_reduce_index<NV>(lane)] = vals[0];
+  __syncthreads();
+  if (tid < R * NT) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < kBgmvThreads / kWave; ++w) s += red[w * NV + tid];
+    vsh[tid] = from_f32<D>(s);  // index g * R + j
+  }
+  __syncthreads();
+  vec8 vv[NT];
+#pragma unroll
+  for (int g = 0; g < NT; ++g) vv[g] = *reinterpret_cast<const vec8*>(vsh + g * R + part * 8);
+
+  // (4) expand, block by block, the next block's y in flight while one is computed
+  auto finish_block = [&](int blk, const vec8(&w)[U], const E(&yv)[U][NT]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float s[NT];
+#pragma unroll
+      for (int g = 0; g < NT; ++g) s[g] = dot8<D>(w[u], vv[g], 0.f);
+#pragma unroll
+      for (int m = CP / 2; m >= 1; m >>= 1)
+#pragma unroll
+        for (int g = 0; g < NT; ++g) s[g] += __shfl_xor(s[g], m, kWave);
+      const int col = column(blk, u);
+      if (part == 0 && col < col_end) {
+#pragma unroll
+        for (int g = 0; g < NT; ++g) yrow[g][col] = accumulate<D>(yv[u][g], s[g] * scale);
+      }
+    }
+  };
+  E ya[U][NT], yb[U][NT];
+  load_y(0, ya);
+#pragma unroll
+  for (int blk = 0; blk < NBLK; blk += 2) {
+    if (col0 + blk * kBlock < col_end) {
+      load_y(blk + 1, yb);
+      __builtin_amdgcn_sched_barrier(0);
+      finish_block(blk, wv[blk], ya);
+      if (blk + 2 < NBLK) load_y(blk + 2, ya);
+      __builtin_amdgcn_sched_barrier(0);
+      finish_block(blk + 1, wv[blk + 1], yb);
+    }
+  }
+}
+
+template <typename D, int R, int U, int NBLK>
+__global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch batch, int h_in,
+                                                                 int64_t layer_idx, float scale) {
+  using E = typename D::E;
+  __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<R * kGroup>::value];
+  __shared__ __attribute__((aligned(16))) E vsh[R * kGroup];
+  const VirtualBlock vb = xcd_virtual_block();
+  const BgmvProblem& P = batch.p[vb.z];
+  const int h_out = P.width;
+  constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
+  const int col0 = vb.x * cols_per_wg;
+  if (col0 >= h_out || vb.y >= P.num_groups) return;
+  const int col_end = min(col0 + cols_per_wg, h_out);
+  const int64_t* rec = P.plan + static_cast<int64_t>(vb.y) * kPlanRecordWords;
+  const int n = static_cast<int>(rec[0]);
+  int toks[kGroup];
+#pragma unroll
+  for (int g = 0; g < kGroup; ++g) toks[g] = static_cast<int>(rec[1 + g]);
+  const E* A = reinterpret_cast<const E*>(rec[5]) + layer_idx * R * static_cast<int64_t>(h_in);
+  const E* B = reinterpret_cast<const E*>(rec[6]) + layer_idx * h_out * static_cast<int64_t>(R);
+  E* Y = static_cast<E*>(P.y);
+  const E* X = static_cast<const E*>(P.x);
+  switch (n) {
+    case 1:
+      bgmv_lora_body<D, R, U, NBLK, 1>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+                                 red, vsh);
+      break;
+    case 2:
+      bgmv_lora_body<D, R, U, NBLK, 2>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+                                 red, vsh);
+      break;
+    case 3:
+      bgmv_lora_body<D, R, U, NBLK, 3>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+                                 red, vsh);
+      break;
+    default:
+      bgmv_lora_body<D, R, U, NBLK, 4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+                                 red, vsh);
       break;
   }
 }
@@ -328,6 +490,27 @@ static hipError_t launch_expand(const BgmvArgs& a, hipStream_t stream) {
   if (chunks <= 4) return launch_expand_cp<D, 4>(a, stream);
   if (chunks <= 8) return launch_expand_cp<D, 8>(a, stream);
   return launch_expand_cp<D, 16>(a, stream);
+}
+
+template <typename D, int R>
+static hipError_t launch_lora_r(const BgmvArgs& a, hipStream_t stream) {
+  // Every column slice of a projection repeats the shrink, so slices are wide: one workgroup
+  // covers 4 expand blocks of 4 columns per lane group (4096 columns at rank 8, 2048 at rank 16)
+  // and holds all their B^T vectors in registers from the start.
+  constexpr int U = 4;
+  constexpr int NBLK = 4;
+  constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
+  dim3 grid((a.wide_max + cols_per_wg - 1) / cols_per_wg, static_cast<unsigned>(a.grid_rows), a.count);
+  hipLaunchKernelGGL((bgmv_lora_kernel<D, R, U, NBLK>), grid, dim3(kBgmvThreads), 0, stream, a.batch, a.h_in,
+                     a.layer_idx, a.scale);
+  return hipGetLastError();
+}
+
+// y += (x A^T) B^T for planned problems of rank 8 or 16 (a.narrow); a.wide_max is the widest h_out.
+hipError_t launch_bgmv_lora(const BgmvArgs& a, hipStream_t stream) {
+  if (a.dtype == LORAX_F16)
+    return a.narrow == 8 ? launch_lora_r<F16, 8>(a, stream) : launch_lora_r<F16, 16>(a, stream);
+  return a.narrow == 8 ? launch_lora_r<BF16, 8>(a, stream) : launch_lora_r<BF16, 16>(a, stream);
 }
 
 hipError_t launch_bgmv(const BgmvArgs& a, hipStream_t stream) {

@@ -93,8 +93,9 @@ int check_common(const void* y, const void* x, const void* w_ptrs, int dtype) {
 }  // namespace
 
 const Tuning& tuning() {
-  static const Tuning t = {env_int("LORAX_BGMV_SHRINK_ROWS"), env_int("LORAX_SHRINK_KSPLIT"),
-                           env_int("LORAX_SHRINK_MB")};
+  static const Tuning t = {env_int("LORAX_BGMV_LORA_BLOCKS"), env_int("LORAX_BGMV_SHRINK_ROWS"), env_int("LORAX_SHRINK_KSPLIT"),
+                           env_int("LORAX_SHRINK_MB"), env_int("LORAX_SHRINK_WAVES"), env_int("LORAX_EXPAND_ROWS"),
+                           env_int("LORAX_SHRINK_NO_ROTATE")};
   return t;
 }
 
@@ -278,6 +279,46 @@ int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32
   a.dtype = dtype;
   const hipError_t e = launch_sgmv_expand(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_expand launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
+int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems, int64_t num_tokens,
+                          int32_t h_in, int32_t r, int64_t layer_idx, float scale, int32_t dtype,
+                          void* stream) {
+  if (num_problems < 0 || num_problems > kMaxBgmvProblems)
+    return fail(LORAX_EINVAL, "num_problems=%d (at most %d per launch)", num_problems, kMaxBgmvProblems);
+  if (num_tokens < 0) return fail(LORAX_EINVAL, "num_tokens=%lld is negative", (long long)num_tokens);
+  if (num_problems == 0 || num_tokens == 0) return LORAX_OK;
+  if (problems == nullptr) return fail(LORAX_EINVAL, "null pointer argument (problems)");
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  if ((r != 8 && r != 16) || h_in <= 0 || h_in % 8 != 0 || h_in >= 65536)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. fused shrink+expand covers rank 8 and 16, h_in=%d r=%d", h_in, r);
+  BgmvArgs a{};
+  a.count = num_problems;
+  a.expand = true;
+  a.narrow = r;
+  a.h_in = h_in;
+  a.num_tokens = num_tokens;
+  a.layer_idx = layer_idx;
+  a.scale = scale;
+  a.accumulate = 1;
+  a.dtype = dtype;
+  for (int i = 0; i < num_problems; ++i) {
+    const lorax_bgmv_problem_t& q = problems[i];
+    if (int rc = check_common(q.y, q.x, q.plan, dtype)) return rc;
+    if (q.num_groups < 0 || q.num_groups > 65535) return fail(LORAX_EINVAL, "num_groups=%d out of range", q.num_groups);
+    if (q.h_out <= 0 || q.h_out % 8 != 0 || q.h_out >= 65536)
+      return fail(LORAX_ENOKERNEL, "No suitable kernel. h_in=%d h_out=%d dtype=%d", h_in, q.h_out, dtype);
+    if (q.y_offset < 0 || q.y_stride < q.y_offset + q.h_out)
+      return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld do not hold h_out=%d columns", (long long)q.y_offset,
+                  (long long)q.y_stride, q.h_out);
+    if (q.num_groups > a.grid_rows) a.grid_rows = q.num_groups;
+    if (q.h_out > a.wide_max) a.wide_max = q.h_out;
+    a.batch.p[i] = BgmvProblem{q.y, q.x, nullptr, nullptr, q.y_offset, q.y_stride, q.h_out, q.plan, q.num_groups};
+  }
+  if (a.grid_rows == 0) return LORAX_OK;
+  const hipError_t e = launch_bgmv_lora(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString(e));
   return LORAX_OK;
 }
 

@@ -16,9 +16,16 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 // Element traits.  E is the 16-bit storage type; vec8 is eight of them (16 bytes).
+// dot2(a, b, c) = c + a.lo * b.lo + a.hi * b.hi on one packed pair of 16-bit elements, fp32
+// accumulate (v_dot2_f32_f16 / v_dot2_f32_bf16): two multiply-adds per instruction and no
+// conversion of the operands, which is what keeps the decode kernels off the vector-ALU limit.
 struct F16 {
   using E = _Float16;
   using vec8 = f16x8;
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    typedef _Float16 pair __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(pair, a), __builtin_bit_cast(pair, b), c, false);
+  }
   static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
@@ -26,6 +33,10 @@ struct F16 {
 struct BF16 {
   using E = __bf16;
   using vec8 = bf16x8;
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    typedef __bf16 pair __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(pair, a), __builtin_bit_cast(pair, b), c, false);
+  }
   static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
@@ -71,6 +82,16 @@ template <typename D>
 __device__ __forceinline__ void store8(typename D::E* p, typename D::vec8 v) {
   *(LORAX_GLOBAL typename D::vec8*)(p) = v;
 }
+// c + sum of the 8 products of two 16-byte vectors.
+template <typename D>
+__device__ __forceinline__ float dot8(typename D::vec8 a, typename D::vec8 b, float c) {
+  const u32x4 ab = __builtin_bit_cast(u32x4, a);
+  const u32x4 bb = __builtin_bit_cast(u32x4, b);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) c = D::dot2(ab[i], bb[i], c);
+  return c;
+}
+
 // v if keep, else zeros - a select on registers, for masking AFTER an unconditional load.
 template <typename D>
 __device__ __forceinline__ typename D::vec8 keep_if(bool keep, typename D::vec8 v) {

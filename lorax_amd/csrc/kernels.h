@@ -36,7 +36,8 @@ struct BgmvArgs {
   int count;          // problems in the batch (grid z)
   bool expand;        // bgmv_impl.cuh:204: h_in < h_out
   int narrow;         // LoRA rank
-  int wide_max;       // shrink: h_in; expand: widest h_out of the batch
+  int wide_max;       // shrink: h_in; expand and fused: widest h_out of the batch
+  int h_in;           // fused shrink+expand only: hidden size of x
   int64_t num_tokens;
   int64_t grid_rows;  // workgroup rows: tokens when chunks are found by scanning, else plan records
   int64_t work_rows;  // estimate of the rows that have work (sizes the rows-per-workgroup choice)
@@ -69,15 +70,20 @@ struct SgmvArgs {
 };
 
 // Launch parameters that can be overridden from the environment for tuning runs
-// (LORAX_BGMV_SHRINK_ROWS, LORAX_SHRINK_KSPLIT, LORAX_SHRINK_MB); 0 = heuristic.
+// (LORAX_BGMV_LORA_BLOCKS, LORAX_BGMV_SHRINK_ROWS, LORAX_SHRINK_KSPLIT, LORAX_SHRINK_MB, LORAX_SHRINK_WAVES, LORAX_EXPAND_ROWS); 0 = heuristic.
 struct Tuning {
+  int bgmv_lora_blocks;
   int bgmv_shrink_rows;
   int shrink_ksplit;
   int shrink_mb;
+  int shrink_waves;
+  int expand_rows;
+  int shrink_no_rotate;
 };
 const Tuning& tuning();
 
 hipError_t launch_bgmv(const BgmvArgs& a, hipStream_t stream);
+hipError_t launch_bgmv_lora(const BgmvArgs& a, hipStream_t stream);
 hipError_t launch_sgmv_shrink(const SgmvArgs& a, hipStream_t stream);
 hipError_t launch_sgmv_expand(const SgmvArgs& a, hipStream_t stream);
 

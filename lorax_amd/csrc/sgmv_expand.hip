@@ -17,16 +17,18 @@
 #include "kernels.h"
 #include "sgmv_tiles.h"
 
+#ifndef LORAX_EXPAND_STAGES
+#define LORAX_EXPAND_STAGES 3
+#endif
+
 namespace lorax {
 
 constexpr int kExpandWaves = 4;
 constexpr int kExpandThreads = kExpandWaves * kWave;
 constexpr int kExpandCols = 64;          // output columns per workgroup
-constexpr int kExpandBlocksPerWave = 4;  // 16-row blocks per wave and tile
-constexpr int kExpandRows = 16 * kExpandWaves * kExpandBlocksPerWave;  // rows per tile
 constexpr int kExpandShortRows = 4;      // row tiles up to this height use the vector path
 constexpr int kPanelPitch = kExpandCols + 4;  // LDS row pitch in elements
-constexpr int kExpandStages = 3;              // register stages of the row-block pipeline
+constexpr int kExpandStages = LORAX_EXPAND_STAGES;  // register stages of the row-block pipeline
 
 // Output column (0..63) that row `a` of the first MFMA operand of accumulator j
 // stands for.  Chosen so that lane group g = a / 4 ends up with columns
@@ -40,7 +42,7 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
     typename D::E* __restrict__ Y, const typename D::E* __restrict__ V,
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int r, int h_out,
-    int64_t y_offset, int64_t y_stride, int64_t layer_idx) {
+    int64_t y_offset, int64_t y_stride, int64_t layer_idx, int rows_per_tile) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   __shared__ __attribute__((aligned(16))) E panel[KS * 32 * kPanelPitch];
@@ -51,11 +53,13 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
   const int wave = tid / kWave;
   const int c = lane & 15;
   const int g = lane >> 4;
+  // Plain numbering on purpose: neighbouring column panels on one XCD (xcd_virtual_block) measured
+  // 30 % slower here - they read adjacent 128-byte pieces of the same rows through the same L2 channels.
   const int n0 = blockIdx.x * kExpandCols;
 
   for (int tile = blockIdx.y;; tile += gridDim.y) {
     RowTile rt;
-    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, kExpandRows, tile, rt)) break;
+    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const E* B = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * r * static_cast<int64_t>(h_out);
     const int nrows = rt.row_end - rt.row0;
     if (nrows <= kExpandShortRows) {
@@ -105,31 +109,7 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
       continue;
     }
 
-    // ---- MFMA path ----
-    // Stage the r x 64 panel of B in LDS (rows k >= r and columns >= h_out as zeros).
-    for (int p = tid; p < KS * 32 * (kExpandCols / 8); p += kExpandThreads) {
-      const int k = p / (kExpandCols / 8);
-      const int cc = (p % (kExpandCols / 8)) * 8;
-      vec8 bv = zero8<D>();
-      if (k < r && n0 + cc < h_out) bv = load8<D>(B + static_cast<int64_t>(k) * h_out + n0 + cc);
-      // rows are 8-byte aligned (pitch 68 elements), so two 8-byte LDS stores
-      const u32x4 bits = __builtin_bit_cast(u32x4, bv);
-      u32x2* dst = reinterpret_cast<u32x2*>(panel + k * kPanelPitch + cc);
-      dst[0] = u32x2{bits[0], bits[1]};
-      dst[1] = u32x2{bits[2], bits[3]};
-    }
-    __syncthreads();
     vec8 bf[4][KS];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int colj = panel_col(j, c);
-#pragma unroll
-      for (int s = 0; s < KS; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) bf[j][s][e] = panel[(s * 32 + g * 8 + e) * kPanelPitch + colj];
-    }
-    __syncthreads();  // the panel may be overwritten by the next tile from here on
-
     const int nmb = (nrows + 15) / 16;
     const bool col_ok0 = n0 + g * 8 < h_out;
     const bool col_ok1 = n0 + 32 + g * 8 < h_out;
@@ -182,12 +162,39 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
     // kExpandStages register stages (static indices, unrolled): the y and v loads of the next
     // kExpandStages-1 blocks are in flight while one block is multiplied and stored.  Surplus
     // trips of the last round re-load the last block and store nothing.
-    if (wave < nmb) {
-      const int n = (nmb - wave + kExpandWaves - 1) / kExpandWaves;
-      auto block_of = [&](int i) { return wave + min(i, n - 1) * kExpandWaves; };
-      vec8 vr[kExpandStages][KS], y0r[kExpandStages], y1r[kExpandStages];
+    // The first y / v loads of the wave's row blocks go out BEFORE the panel of B is staged: they do
+    // not depend on it, so the tile's first memory round trip overlaps the operand set-up.
+    const int n = wave < nmb ? (nmb - wave + kExpandWaves - 1) / kExpandWaves : 0;
+    auto block_of = [&](int i) { return wave + min(i, max(n, 1) - 1) * kExpandWaves; };
+    vec8 vr[kExpandStages][KS], y0r[kExpandStages], y1r[kExpandStages];
 #pragma unroll
-      for (int s = 0; s < kExpandStages - 1; ++s) load_block(block_of(s), vr[s], y0r[s], y1r[s]);
+    for (int s = 0; s < kExpandStages - 1; ++s) load_block(block_of(s), vr[s], y0r[s], y1r[s]);
+
+    // ---- MFMA path ----
+    // Stage the r x 64 panel of B in LDS (rows k >= r and columns >= h_out as zeros).
+    for (int p = tid; p < KS * 32 * (kExpandCols / 8); p += kExpandThreads) {
+      const int k = p / (kExpandCols / 8);
+      const int cc = (p % (kExpandCols / 8)) * 8;
+      vec8 bv = zero8<D>();
+      if (k < r && n0 + cc < h_out) bv = load8<D>(B + static_cast<int64_t>(k) * h_out + n0 + cc);
+      // rows are 8-byte aligned (pitch 68 elements), so two 8-byte LDS stores
+      const u32x4 bits = __builtin_bit_cast(u32x4, bv);
+      u32x2* dst = reinterpret_cast<u32x2*>(panel + k * kPanelPitch + cc);
+      dst[0] = u32x2{bits[0], bits[1]};
+      dst[1] = u32x2{bits[2], bits[3]};
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int colj = panel_col(j, c);
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bf[j][s][e] = panel[(s * 32 + g * 8 + e) * kPanelPitch + colj];
+    }
+    __syncthreads();  // the panel may be overwritten by the next tile from here on
+
+    if (n > 0) {
       for (int i = 0; i < n; i += kExpandStages) {
 #pragma unroll
         for (int s = 0; s < kExpandStages; ++s) {
@@ -204,13 +211,17 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
 
 template <typename D, int KS>
 static hipError_t launch_expand_ks(const SgmvArgs& a, hipStream_t stream) {
-  const int64_t tiles = (a.num_tokens + kExpandRows - 1) / kExpandRows + a.num_segments;
+  // Rows per tile: the tile prologue (tile search, staging and transposing the panel of B) is
+  // amortised over the tile's rows, so tiles are tall when there are many rows to go round.
+  int rows_per_tile = a.num_tokens >= 8192 ? 512 : 256;
+  if (tuning().expand_rows > 0) rows_per_tile = (tuning().expand_rows + 63) / 64 * 64;
+  const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
   dim3 grid((a.d_out + kExpandCols - 1) / kExpandCols,
             static_cast<unsigned>(tiles < 65535 ? tiles : 65535));
   hipLaunchKernelGGL((sgmv_expand_kernel<D, KS>), grid, dim3(kExpandThreads), 0, stream,
                      static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x),
                      a.w_ptrs, a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens),
-                     a.d_in, a.d_out, a.y_offset, a.y_stride, a.layer_idx);
+                     a.d_in, a.d_out, a.y_offset, a.y_stride, a.layer_idx, rows_per_tile);
   return hipGetLastError();
 }
 

@@ -25,14 +25,17 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in,
     int64_t layer_idx, int ksplit, float* __restrict__ partials,
-    uint32_t* __restrict__ counters, int num_counters) {
+    uint32_t* __restrict__ counters, int num_counters, int rotate_k) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   constexpr int R = NB * 16;
   constexpr int ROWS = MB * 16;
   constexpr int THREADS = WAVES * kWave;
   // register stages of the K pipeline: as many as fit next to the accumulators
-  constexpr int STAGES = (MB + NB) * 4 * 4 + MB * NB * 4 <= 200 ? 4 : ((MB + NB) * 4 * 3 + MB * NB * 4 <= 232 ? 3 : 2);
+  constexpr int kBudget = WAVES >= 16 ? 96 : (WAVES >= 8 ? 200 : 232);  // registers for stages + accumulators
+  constexpr int STAGES = (MB + NB) * 4 * 4 + MB * NB * 4 <= kBudget - 32
+                             ? 4
+                             : ((MB + NB) * 4 * 3 + MB * NB * 4 <= kBudget ? 3 : 2);
   __shared__ f32x4 red[WAVES][NB][kWave];
   __shared__ uint32_t arrival;
 
@@ -41,14 +44,17 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
   const int wave = tid / kWave;
   const int c = lane & 15;   // operand row inside a 16-row block
   const int g = lane >> 4;   // which 8 of the 32 k of a step
-  const int kc = blockIdx.x;
+  // XCD-aware numbering: consecutive row tiles (the tiles of one segment) run on one XCD, so the
+  // segment's A is fetched into one L2 instead of into every L2 that happens to get a tile.
+  const VirtualBlock vb = xcd_virtual_block();
+  const int kc = vb.x;
 
   const int ksteps = (h_in + 31) / 32;
   const int per = (ksteps + ksplit - 1) / ksplit;
   const int ks0 = kc * per;
   const int ks1 = min(ks0 + per, ksteps);
 
-  for (int tile = blockIdx.y;; tile += gridDim.y) {
+  for (int tile = vb.y;; tile += gridDim.y) {
     RowTile rt;
     if (!find_row_tile(s_start, s_end, num_segments, num_tokens, ROWS, tile, rt)) break;
     // Disjoint segments never produce this many tiles (the host sizes ksplit for that);
@@ -99,7 +105,14 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
     const int first = ks0 + wave;
     if (first < last) {
       const int n = (last - first + WAVES - 1) / WAVES;
-      auto step_ks = [&](int i) { return first + min(i, n - 1) * WAVES; };
+      // Rows of x are a power-of-two number of bytes apart, so workgroups that all start at k = 0
+      // and advance in step keep hitting the same few HBM channels.  Every tile therefore starts
+      // its walk over K at a different step and wraps around (the sum does not care about order).
+      const int rot = static_cast<int>((static_cast<unsigned>(tile) * 2654435761u) >> 8) % n;
+      auto step_ks = [&](int i) {
+        const int j = min(i, n - 1) + (rotate_k ? rot : 0);
+        return first + (j >= n ? j - n : j) * WAVES;
+      };
       vec8 xr[STAGES][MB], wr[STAGES][NB];
 #pragma unroll
       for (int s = 0; s < STAGES - 1; ++s) load_step(step_ks(s), xr[s], wr[s]);
@@ -251,17 +264,26 @@ __global__ __launch_bounds__(256) void sgmv_shrink_hr_kernel(
 // ---------------------------------------------------------------------------------
 // Host-side launchers
 // ---------------------------------------------------------------------------------
-template <typename D, int NB, int MB>
-static hipError_t launch_rh(const SgmvArgs& a, int ksplit, hipStream_t stream) {
-  constexpr int WAVES = 4;
+template <typename D, int NB, int MB, int WAVES>
+static hipError_t launch_rh_w(const SgmvArgs& a, int ksplit, hipStream_t stream) {
   const int64_t tiles = (a.num_tokens + MB * 16 - 1) / (MB * 16) + a.num_segments;
   dim3 grid(ksplit, static_cast<unsigned>(tiles < 65535 ? tiles : 65535));
   hipLaunchKernelGGL((sgmv_shrink_rh_kernel<D, NB, MB, WAVES>), grid, dim3(WAVES * kWave), 0,
                      stream, static_cast<typename D::E*>(a.y),
                      static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end,
                      a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, ksplit,
-                     a.partials, a.counters, static_cast<int>(a.num_counters));
+                     a.partials, a.counters, static_cast<int>(a.num_counters), tuning().shrink_no_rotate ? 0 : 1);
   return hipGetLastError();
+}
+
+// Waves per workgroup = how many ways K is split inside the workgroup (through LDS, no fences).
+template <typename D, int NB, int MB>
+static hipError_t launch_rh(const SgmvArgs& a, int ksplit, hipStream_t stream) {
+  int waves = 4;
+  if (tuning().shrink_waves > 0) waves = tuning().shrink_waves;
+  if (waves >= 16) return launch_rh_w<D, NB, MB, 16>(a, ksplit, stream);
+  if (waves >= 8) return launch_rh_w<D, NB, MB, 8>(a, ksplit, stream);
+  return launch_rh_w<D, NB, MB, 4>(a, ksplit, stream);
 }
 
 template <typename D, int NB>

@@ -105,6 +105,15 @@ class LoraLinear(nn.Module):
 
         step = _native.MAX_BGMV_PROBLEMS
         for r, jobs in decode_jobs.items():
+            if not tensor_parallel:
+                # small slabs: shrink and expand in one launch, v never leaves the chip
+                single = [j for j in jobs if j[0].plan is not None and _native.bgmv_lora_fits(r, input.size(1), j[2])]
+                jobs = [j for j in jobs if not any(j is s for s in single)]
+                for i in range(0, len(single), step):
+                    _native.bgmv_lora_multi(
+                        [(result, input, rs.plan, start, width) for rs, start, width in single[i : i + step]],
+                        r, self.layer_id,
+                    )
             for i in range(0, len(jobs), step):
                 chunk = jobs[i : i + step]
                 # v needs no zero-fill: the shrink overwrites the rows of routed tokens and the

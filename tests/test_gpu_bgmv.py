@@ -234,3 +234,41 @@ def test_bgmv_multi_matches_separate_launches(r):
         _native.bgmv_multi([shrink[0], (torch.zeros((T, r + 8), dtype=dtype, device=DEV),) + shrink[1][1:]], 1)
     with pytest.raises(RuntimeError, match="between 1 and 4"):
         _native.bgmv_multi(shrink + shrink, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("r", [8, 16])
+@pytest.mark.parametrize("h_in,sizes", [(4096, [4096, 1024, 1024]), (2752, [1152]), (14336, [4096])])
+def test_bgmv_single_launch_shrink_expand(dtype, r, h_in, sizes):
+    """lorax_bgmv_lora_multi (shrink + expand in one launch, v on chip) against the two-step oracle."""
+    from lorax_amd import _native
+    from lorax_amd.adapters import build_bgmv_plan
+
+    print(f"case dtype={dtype} r={r} h_in={h_in} sizes={sizes}", flush=True)
+    T, n = 77, 9
+    gen = torch.Generator().manual_seed(5 * r + h_in)
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    y0 = randn((T, sum(sizes)), 0.5, gen, dtype, DEV)
+    y = y0.clone()
+    y_ref = y0.cpu().clone()
+    problems, keep_alive = [], []
+    off = 0
+    for h_out in sizes:
+        wa_t = _stacks(n, 2, r, h_in, gen, dtype)
+        wb_t = _stacks(n, 2, h_out, r, gen, dtype)
+        keep_alive.append((wa_t, wb_t))
+        idx = _indices(T, n, gen, drop=0.15)
+        records = build_bgmv_plan(idx.tolist(), [w.data_ptr() for w in wa_t], [w.data_ptr() for w in wb_t])
+        plan = torch.tensor(records, dtype=torch.int64, device=DEV).reshape(-1, 8)
+        problems.append((y, x, plan, off, h_out))
+        v_ref = torch.zeros((T, r), dtype=dtype)
+        O.bgmv_ref(v_ref, x.cpu(), [w.cpu() for w in wa_t], idx.tolist(), 1)
+        part = y_ref[:, off:off + h_out].clone()
+        O.bgmv_ref(part, v_ref, [w.cpu() for w in wb_t], idx.tolist(), 1)
+        y_ref[:, off:off + h_out] = part
+        off += h_out
+    _native.bgmv_lora_multi(problems, r, 1)
+    torch.cuda.synchronize()
+    assert_close(y, y_ref, "single-launch LoRA")
+    with pytest.raises(RuntimeError, match="No suitable kernel"):
+        _native.bgmv_lora_multi(problems, 32, 1)
