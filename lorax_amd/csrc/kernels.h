@@ -79,6 +79,8 @@ struct Tuning {
   int shrink_waves;
   int expand_rows;
   int shrink_no_rotate;
+  int shrink_lds;  // LORAX_SHRINK_LDS: 1 = always take the LDS-staged shrink where it applies, -1 = never
+  int shrink_lds_kb;  // LORAX_SHRINK_LDS_KB: LDS budget of the staged shrink's buffers
 };
 const Tuning& tuning();
 
@@ -86,6 +88,9 @@ hipError_t launch_bgmv(const BgmvArgs& a, hipStream_t stream);
 hipError_t launch_bgmv_lora(const BgmvArgs& a, hipStream_t stream);
 hipError_t launch_sgmv_shrink(const SgmvArgs& a, hipStream_t stream);
 hipError_t launch_sgmv_expand(const SgmvArgs& a, hipStream_t stream);
+// LDS-staged shrink (sgmv_shrink_lds.hip): [L, r, h_in] layout, h_in a multiple of 128.
+bool sgmv_shrink_lds_applies(const SgmvArgs& a);
+hipError_t launch_sgmv_shrink_lds(const SgmvArgs& a, hipStream_t stream);
 
 // Workspace layout constants shared by capi.hip and sgmv_shrink.hip.
 constexpr size_t kPartialBytes = 96u << 20;  // fp32 split-K partial sums

@@ -360,6 +360,9 @@ static hipError_t launch_shrink_dtype(const SgmvArgs& a, hipStream_t stream) {
 }
 
 hipError_t launch_sgmv_shrink(const SgmvArgs& a, hipStream_t stream) {
+  // The LDS-staged kernel is the faster one wherever it applies (h_in a multiple of 128).
+  if (tuning().shrink_lds >= 0 && sgmv_shrink_lds_applies(a))
+    return launch_sgmv_shrink_lds(a, stream);
   return a.dtype == LORAX_F16 ? launch_shrink_dtype<F16>(a, stream)
                               : launch_shrink_dtype<BF16>(a, stream);
 }

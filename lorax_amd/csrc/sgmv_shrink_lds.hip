@@ -1,0 +1,302 @@
+// SGMV shrink, LDS-staged variant for the [L, r, h_in] layout and hidden sizes that are a
+// multiple of 128: v[s:e, :r] += T(x[s:e, :] @ A_i^T).
+//
+// Why it exists: in the register-only kernel (sgmv_shrink.hip) every wave instruction reads
+// 16 rows x 64 bytes, rows a power-of-two number of bytes apart, and every wave fetches its own
+// copy of the A fragments through L1.  Measured with the arithmetic removed, x alone streams at
+// 3.3-3.7 TB/s in that pattern against 5.4-5.7 TB/s for contiguous 1 KB reads, and adding the
+// (fully L2-resident) A fragments costs another 60 %: the L2 -> L1 path, not HBM and not the
+// MFMAs, bounds that kernel.  Here a workgroup stages x and A tiles in LDS with direct-to-LDS
+// loads (global_load_lds_dwordx4: 64 lanes x 16 B per instruction, four 256-byte row pieces), A
+// is fetched once per workgroup instead of once per wave, and the MFMA operands come from LDS.
+//
+// Layout of one stage in LDS: x tile [ROWS][128 k] then A tile [R][128 k], rows of 256 bytes = 16
+// chunks of 16 bytes; chunk q of row i is stored at position q ^ (i & 15), so the 16 lanes of one
+// ds_read_b128 group (same chunk, 16 consecutive rows) hit 16 different bank groups - no padding,
+// which direct-to-LDS loads could not produce anyway (a wave instruction writes 1 KB contiguously).
+//
+// Pipeline: STAGES buffers; the loads of the next STAGES-1 stages are in flight while one stage is
+// multiplied.  Per K step one s_waitcnt vmcnt(N) (the wave's own loads of that stage have landed)
+// and one s_barrier (everybody's have; everybody is done with the buffer about to be refilled).
+// The barrier is a bare s_barrier: __syncthreads() would wait for ALL outstanding loads and
+// serialise the pipeline.
+#include "kernels.h"
+#include "sgmv_tiles.h"
+
+namespace lorax {
+
+constexpr int kLdsKc = 128;             // k elements per stage
+constexpr int kLdsRowBytes = kLdsKc * 2;
+constexpr int kLdsThreads = 256;
+constexpr int kLdsMaxStages = 8;
+constexpr int kLdsMaxBytes = 156 * 1024;  // of the CU's 160 KB
+
+#define LORAX_LDS __attribute__((address_space(3)))
+
+// s_waitcnt vmcnt(N), N a compile-time constant (gfx9 encoding: vmcnt = simm16[3:0] | simm16[15:14] << 4)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  constexpr int n = N < 63 ? N : 63;  // 6-bit counter; waiting for fewer outstanding loads is always safe
+  __builtin_amdgcn_s_waitcnt((n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// Waits until at most `pending` groups of LOADS loads (the younger stages) are outstanding.
+template <int LOADS>
+__device__ __forceinline__ void wait_pending(int pending) {
+  switch (pending) {
+    case 0: wait_vmcnt<0>(); break;
+    case 1: wait_vmcnt<LOADS>(); break;
+    case 2: wait_vmcnt<2 * LOADS>(); break;
+    case 3: wait_vmcnt<3 * LOADS>(); break;
+    case 4: wait_vmcnt<4 * LOADS>(); break;
+    case 5: wait_vmcnt<5 * LOADS>(); break;
+    default: wait_vmcnt<6 * LOADS>(); break;
+  }
+}
+
+template <typename D, int NB, int MBLK, bool KSPLIT>
+__global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
+    typename D::E* __restrict__ V, const typename D::E* __restrict__ X,
+    const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
+    const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in,
+    int64_t layer_idx, int stages) {
+  using E = typename D::E;
+  using vec8 = typename D::vec8;
+  constexpr int R = NB * 16;
+  constexpr int ROWS = MBLK * 16;
+  constexpr int kXBytes = ROWS * kLdsRowBytes;
+  constexpr int kABytes = R * kLdsRowBytes;
+  constexpr int kStageBytes = kXBytes + kABytes;
+  constexpr int kXLoads = MBLK;  // 16-byte loads per thread and stage for x: ROWS * 16 chunks / 256 threads
+  constexpr int kALoads = NB;
+  constexpr int kLoads = kXLoads + kALoads;
+  // Work split among the four waves.  KSPLIT: each wave multiplies one 32-wide k slice of every
+  // stage for all blocks of the tile and the partial sums are added through LDS at the end (every
+  // staged byte is read from LDS once).  Otherwise: waves as WM x WN over the (row block, rank
+  // block) grid, each with its own output blocks and all k.
+  constexpr int WN = KSPLIT ? 1 : ((NB % 2 == 0) ? 2 : 1);
+  constexpr int WM = KSPLIT ? 1 : 4 / WN;
+  static_assert(MBLK % WM == 0, "row blocks must divide among the waves");
+  static_assert(!KSPLIT || 4 * MBLK * NB * 1024 <= 2 * kStageBytes, "partial sums must fit in two stage buffers");
+  constexpr int MPW = MBLK / WM;  // row blocks per wave
+  constexpr int NPW = NB / WN;    // rank blocks per wave
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int c = lane & 15;
+  const int g = lane >> 4;
+  const int wm = KSPLIT ? 0 : wave % WM;
+  const int wn = KSPLIT ? 0 : wave / WM;
+  const VirtualBlock vb = xcd_virtual_block();
+  const int nst = h_in / kLdsKc;
+
+  for (int tile = vb.x;; tile += gridDim.x) {
+    RowTile rt;
+    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, ROWS, tile, rt)) break;
+    const E* A = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * R * static_cast<int64_t>(h_in);
+
+    // Source addresses of this thread's chunks.  Load j of a thread covers chunk id j * 256 + tid of
+    // the tile: row = id / 16, position = id % 16, and it fetches the row's chunk position ^ (row & 15).
+    const E* xsrc[kXLoads];
+    const E* asrc[kALoads];
+#pragma unroll
+    for (int j = 0; j < kXLoads; ++j) {
+      const int id = j * kLdsThreads + tid;
+      const int row = id >> 4;
+      const int grow = min(rt.row0 + row, rt.row_end - 1);  // rows past the tile re-read its last row
+      xsrc[j] = X + static_cast<int64_t>(grow) * h_in + (((id & 15) ^ (row & 15)) << 3);
+    }
+#pragma unroll
+    for (int j = 0; j < kALoads; ++j) {
+      const int id = j * kLdsThreads + tid;
+      const int row = id >> 4;
+      asrc[j] = A + static_cast<int64_t>(row) * h_in + (((id & 15) ^ (row & 15)) << 3);
+    }
+    auto issue = [&](int st, int slot) {
+      char* buf = lds + slot * kStageBytes;
+      const int k = st * kLdsKc;
+#pragma unroll
+      for (int j = 0; j < kXLoads; ++j)
+        __builtin_amdgcn_global_load_lds((const LORAX_GLOBAL void*)(xsrc[j] + k),
+                                         (LORAX_LDS void*)(buf + (j * kLdsThreads + wave * kWave) * 16), 16, 0, 0);
+#pragma unroll
+      for (int j = 0; j < kALoads; ++j)
+        __builtin_amdgcn_global_load_lds((const LORAX_GLOBAL void*)(asrc[j] + k),
+                                         (LORAX_LDS void*)(buf + kXBytes + (j * kLdsThreads + wave * kWave) * 16), 16,
+                                         0, 0);
+    };
+
+    f32x4 acc[MPW][NPW];
+#pragma unroll
+    for (int mb = 0; mb < MPW; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < NPW; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // all waves must be done reading the previous tile's buffers before they are refilled
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    for (int s = 0; s < stages - 1; ++s)
+      if (s < nst) issue(s, s);
+
+    int slot = 0;            // buffer holding stage st
+    int fill = stages - 1;   // buffer the next issued stage goes to
+    for (int st = 0; st < nst; ++st) {
+      // the loads of stage st were issued stages-1 steps ago; up to stages-2 later stages are pending
+      wait_pending<kLoads>(min(stages - 2, nst - 1 - st));
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (st + stages - 1 < nst) issue(st + stages - 1, fill);
+      const char* xb = lds + slot * kStageBytes;
+      const char* ab = xb + kXBytes;
+      slot = slot + 1 == stages ? 0 : slot + 1;
+      fill = fill + 1 == stages ? 0 : fill + 1;
+#pragma unroll
+      for (int jj = 0; jj < (KSPLIT ? 1 : kLdsKc / 32); ++jj) {
+        const int j = KSPLIT ? wave : jj;
+        const int q = ((j * 4 + g) ^ c) * 16;  // swizzled chunk position of this lane's 8 k
+        vec8 xf[MPW], af[NPW];
+#pragma unroll
+        for (int mb = 0; mb < MPW; ++mb)
+          xf[mb] = *reinterpret_cast<const vec8*>(xb + ((wm * MPW + mb) * 16 + c) * kLdsRowBytes + q);
+#pragma unroll
+        for (int nb = 0; nb < NPW; ++nb)
+          af[nb] = *reinterpret_cast<const vec8*>(ab + ((wn * NPW + nb) * 16 + c) * kLdsRowBytes + q);
+#pragma unroll
+        for (int mb = 0; mb < MPW; ++mb)
+#pragma unroll
+          for (int nb = 0; nb < NPW; ++nb) acc[mb][nb] = D::mfma16(af[nb], xf[mb], acc[mb][nb]);
+      }
+    }
+
+    // acc[mb][nb][i] of lane (g, c) is D[n = nblock*16 + 4g + i][row = mblock*16 + c].
+    if constexpr (KSPLIT) {
+      // Partial sums of the four waves meet in LDS (the stage buffers are free: the last stage was
+      // waited for with no load outstanding), then the 256 threads share the blocks' elements.
+      f32x4* red = reinterpret_cast<f32x4*>(lds);
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+      for (int mb = 0; mb < MBLK; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) red[(wave * MBLK * NB + mb * NB + nb) * kWave + lane] = acc[mb][nb];
+      __syncthreads();
+      for (int i = tid; i < MBLK * NB * kWave; i += kLdsThreads) {
+        const int blk = i / kWave, l = i % kWave;
+        f32x4 sum = red[i];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+          const f32x4 part = red[w * MBLK * NB * kWave + i];
+          sum[0] += part[0]; sum[1] += part[1]; sum[2] += part[2]; sum[3] += part[3];
+        }
+        const int row = rt.row0 + (blk / NB) * 16 + (l & 15);
+        if (row < rt.row_end) accumulate4<D>(V + static_cast<int64_t>(row) * R + (blk % NB) * 16 + 4 * (l >> 4), sum);
+      }
+    } else {
+      // every wave owns its output blocks: no cross-wave reduction
+#pragma unroll
+      for (int mb = 0; mb < MPW; ++mb) {
+        const int row = rt.row0 + (wm * MPW + mb) * 16 + c;
+        if (row < rt.row_end) {
+#pragma unroll
+          for (int nb = 0; nb < NPW; ++nb)
+            accumulate4<D>(V + static_cast<int64_t>(row) * R + (wn * NPW + nb) * 16 + 4 * g, acc[mb][nb]);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------
+template <typename D, int NB, int MBLK, bool KSPLIT>
+static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
+  constexpr int kStageBytes = (MBLK + NB) * 16 * kLdsRowBytes;
+  const int64_t tiles = (a.num_tokens + MBLK * 16 - 1) / (MBLK * 16) + a.num_segments;
+  // Stage buffers: all of a CU's LDS when there is at most one workgroup per CU; a third of it when the
+  // tiles make one to three rounds over the CUs (more resident workgroups even out the last round);
+  // half of it for long launches.  2 to 8 stages.
+  int budget = tiles <= 256 ? 150 * 1024 : (tiles <= 768 ? 50 * 1024 : 76 * 1024);
+  if (tuning().shrink_lds_kb > 0) budget = tuning().shrink_lds_kb * 1024;
+  int stages = budget / kStageBytes;
+  stages = stages < 2 ? 2 : (stages > kLdsMaxStages ? kLdsMaxStages : stages);
+  static_assert(2 * kStageBytes <= kLdsMaxBytes, "two stages must fit in LDS");
+  while (stages * kStageBytes > kLdsMaxBytes) --stages;
+  const int lds_bytes = stages * kStageBytes;
+  auto kernel = sgmv_shrink_lds_kernel<D, NB, MBLK, KSPLIT>;
+  // Raising the dynamic LDS limit is needed once per kernel and device.
+  static bool configured[64] = {};
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  if (device < 0 || device >= 64 || !configured[device]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kLdsMaxBytes);
+    if (e != hipSuccess) return e;
+    if (device >= 0 && device < 64) configured[device] = true;
+  }
+  dim3 grid(static_cast<unsigned>(tiles < (1 << 20) ? tiles : (1 << 20)));
+  hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, static_cast<typename D::E*>(a.y),
+                     static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end, a.num_segments,
+                     static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages);
+  return hipGetLastError();
+}
+
+template <typename D, int NB>
+static hipError_t launch_lds_nb(const SgmvArgs& a, hipStream_t stream) {
+  // Row-tile height: the tallest of 64 / 32 / 16 rows that still yields 128 tiles (a workgroup streams
+  // about 50 GB/s, so fewer, larger tiles leave HBM idle) and is not much taller than the average
+  // segment (rows past a segment's end are padding).  Short tiles re-read A more often, but from L2.
+  const int64_t avg_len = a.num_tokens / (a.num_segments > 0 ? a.num_segments : 1);
+  int mblk = 4;
+  while (mblk > 1 && ((a.num_tokens + mblk * 16 - 1) / (mblk * 16) + a.num_segments < 128 || mblk * 8 > avg_len))
+    mblk /= 2;
+  if (tuning().shrink_mb > 0) mblk = tuning().shrink_mb;
+  const bool ksplit = tuning().shrink_lds != 2;
+  if (mblk >= 4) {
+    if constexpr (NB <= 4) {
+      if (ksplit) return launch_lds_m<D, NB, 4, true>(a, stream);
+    }
+    return launch_lds_m<D, NB, 4, false>(a, stream);
+  }
+  if (mblk == 2) {
+    if constexpr (NB % 2 == 0) {
+      if (!ksplit) return launch_lds_m<D, NB, 2, false>(a, stream);
+    }
+    return launch_lds_m<D, NB, 2, true>(a, stream);
+  }
+  return launch_lds_m<D, NB, 1, true>(a, stream);
+}
+
+template <typename D>
+static hipError_t launch_lds_dtype(const SgmvArgs& a, hipStream_t stream) {
+  switch (a.d_out / 16) {
+    case 1:
+      return launch_lds_nb<D, 1>(a, stream);
+    case 2:
+      return launch_lds_nb<D, 2>(a, stream);
+    case 3:
+      return launch_lds_nb<D, 3>(a, stream);
+    case 4:
+      return launch_lds_nb<D, 4>(a, stream);
+    case 5:
+      return launch_lds_nb<D, 5>(a, stream);
+    case 6:
+      return launch_lds_nb<D, 6>(a, stream);
+    case 7:
+      return launch_lds_nb<D, 7>(a, stream);
+    case 8:
+      return launch_lds_nb<D, 8>(a, stream);
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+bool sgmv_shrink_lds_applies(const SgmvArgs& a) {
+  return a.a_layout == LORAX_A_RH && a.d_in % kLdsKc == 0 && a.d_out % 16 == 0 && a.d_out >= 16 && a.d_out <= 128;
+}
+
+hipError_t launch_sgmv_shrink_lds(const SgmvArgs& a, hipStream_t stream) {
+  return a.dtype == LORAX_F16 ? launch_lds_dtype<F16>(a, stream) : launch_lds_dtype<BF16>(a, stream);
+}
+
+}  // namespace lorax

@@ -124,6 +124,40 @@ def test_sgmv_shrink_expand_vs_oracle(dtype, r, h_in, h_out, lens):
     assert torch.count_nonzero(v.cpu()[~covered]) == 0
 
 
+@pytest.mark.parametrize("r,h_in,lens", [
+    # the shrink launcher picks its tile height from the row and segment counts and its kernel family from
+    # the rank and from h_in % 128; these shapes reach every combination it has
+    (16, 256, [3000, 1, 2500, 2691]),         # 64-row tiles
+    (64, 384, [4096, 4096]),                  # 64-row tiles, four rank blocks
+    (128, 256, [2048, 2048, 2048, 2048]),     # 64-row tiles, rank 128
+    (96, 128, [2100, 2100, 2100, 2100]),      # 64-row tiles, odd number of rank blocks above four
+    (32, 512, [500] * 8 + [5]),               # 32-row tiles
+    (48, 256, [600, 700, 800, 900, 1000]),    # 32-row tiles, odd number of rank blocks
+    (128, 256, [40] * 100 + [1] * 60),        # 32-row tiles, rank 128, many short segments
+    (16, 128, [1] * 200),                     # 16-row tiles, one row each
+    (64, 192, [3000, 2000, 3000]),            # h_in not a multiple of 128: register-operand kernel
+    (16, 4160, [100, 28]),                    # the same with K split across workgroups
+])
+def test_sgmv_shrink_tile_variants(r, h_in, lens):
+    print(f"case r={r} h_in={h_in} segments={len(lens)} rows={sum(lens)}", flush=True)
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(r + h_in + len(lens))
+    T, x, y0, wa, wb, starts, ends = _ragged_case(dtype, r, h_in, 128, lens, gen, L=2)
+    y = y0.clone()
+    v = _run_pair(x, y, wa, wb, starts, ends, 1, r)
+    torch.cuda.synchronize()
+    cpu = lambda ts: [t.cpu() if t is not None else None for t in ts]  # noqa: E731
+    v_ref = O.sgmv_ref(torch.zeros((T, r), dtype=dtype), x.cpu(), cpu(wa),
+                       [torch.eye(r, dtype=dtype).expand(2, r, r) for _ in wb], starts, ends, 1, r)
+    y_ref = O.sgmv_ref(y0.cpu().clone(), x.cpu(), cpu(wa), cpu(wb), starts, ends, 1, r)
+    assert_close(v, v_ref, "shrink output v")
+    assert_close(y, y_ref, "expand output y")
+    covered = torch.zeros(T, dtype=torch.bool)
+    for s, e in zip(starts, ends):
+        covered[s:e] = True
+    assert torch.count_nonzero(v.cpu()[~covered]) == 0
+
+
 @pytest.mark.parametrize("r", [48, 80, 96, 112])
 def test_sgmv_other_multiples_of_16(r):
     """pad_to_min_rank can produce these ranks (punica.py:57-65); the reference's shrink has no
