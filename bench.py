@@ -77,6 +77,7 @@ class Plan:
         from lorax_amd.adapters import LORA
 
         self.w = w
+        self.pattern = pattern
         self.use_plan = use_plan
         self.fuse_small_ranks = fuse_small_ranks
         self.batch = w.batch_data()
@@ -138,8 +139,13 @@ class Plan:
             else:
                 sgmv._kernels.sgmv_cutlass(v, x, a_ptr, starts, ends, tmp_s, layer)
 
+        bt_ptr = rd.lora_b_t_ptr if self.pattern == "fused" else None
+
         def expand(layer):
-            sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_ptr, starts, ends, layer, off, size)
+            if bt_ptr is not None:
+                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, bt_ptr, starts, ends, layer, off, size, transposed=True)
+            else:
+                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_ptr, starts, ends, layer, off, size)
 
         self.calls.append(("zero", lambda layer: v.zero_(), 0, 0))
         self.calls.append(("sgmv_shrink", shrink, rows * h_in * e + uniq * r * h_in * e + rows * r * e,

@@ -47,6 +47,15 @@ extern "C" {
 #define LORAX_A_RH 0
 #define LORAX_A_HR 1
 
+/* B layouts accepted by lorax_sgmv_expand (one adapter's stack, row-major):
+ *   LORAX_B_RH: [num_layers, r, h_out] - what the reference's cutlass grouped GEMM reads
+ *                                        (sgmv_cutlass.cuh:46-47; adapters/lora.py:274-281)
+ *   LORAX_B_HR: [num_layers, h_out, r] - the transposed stack the reference keeps for BGMV decode
+ *                                        (adapters/lora.py:117-126, weights_b_t); the faster
+ *                                        one here: a column panel is one contiguous run      */
+#define LORAX_B_RH 0
+#define LORAX_B_HR 1
+
 /* Size in bytes of the shrink scratch the reference API passes around
  * (lorax_server/utils/punica.py:145-147; checked at punica_ops.cc:389-390). */
 #define LORAX_SHRINK_TMP_BYTES (8 * 1024 * 1024)
@@ -152,15 +161,16 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
  * sgmv/sgmv_cutlass.cuh:86-131).
  *
  *   for every segment i with s_end[i] > s_start[i]:
- *     B = (dtype*)w_ptrs[i] + layer_idx * r * h_out                  // [r, h_out]
+ *     B = (dtype*)w_ptrs[i] + layer_idx * r * h_out                  // [r, h_out] (LORAX_B_RH)
  *     y[s:e, y_offset : y_offset + h_out] += dtype(v[s:e, :] @ B)    // row pitch y_stride
+ *   With b_layout = LORAX_B_HR the stack holds B^T, [h_out, r] per layer, and the result is the same.
  *
  * r must be a multiple of 8 in [8, 128]; h_out, y_offset and y_stride multiples of 8.
  */
 int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
-                      int32_t h_out, int64_t y_offset, int64_t y_stride, int64_t layer_idx,
-                      void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
+                      int32_t h_out, int32_t b_layout, int64_t y_offset, int64_t y_stride,
+                      int64_t layer_idx, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
 
 /* Bytes of grouped-GEMM argument scratch for `num_problems` segments.  Replaces
  * sgmv_tmp_size (sgmv/sgmv_cutlass.cuh:54-58): 3 pointers + 3 int64 + one

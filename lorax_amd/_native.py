@@ -19,6 +19,7 @@ LIB_PATH = Path(__file__).resolve().parent / "liblorax_hip.so"
 
 F16, BF16 = 0, 1
 A_RH, A_HR = 0, 1
+B_RH, B_HR = 0, 1
 SHRINK_TMP_BYTES = 8 * 1024 * 1024
 
 _c = ctypes
@@ -67,7 +68,7 @@ _SIGNATURES = {
     "lorax_sgmv_expand": (
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
-         _c.c_int32, _c.c_int32, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
+         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
          _c.c_int32, _c.c_void_p],
     ),
     "lorax_sgmv_tmp_size": (_c.c_size_t, [_c.c_int32]),
@@ -317,14 +318,17 @@ def _check_sgmv(y, x, w_ptr, s_start, s_end, tmp) -> None:
         raise RuntimeError(f"CHECK_EQ(y.size(0), x.size(0)) failed. {y.size(0)} vs {x.size(0)}")
 
 
-def sgmv_expand(y, x, w_ptr, s_start, s_end, tmp, layer_idx, y_offset=0, y_slice_size=None) -> None:
-    """lorax_sgmv_expand with an optional column window of y."""
+def sgmv_expand(y, x, w_ptr, s_start, s_end, tmp, layer_idx, y_offset=0, y_slice_size=None,
+                transposed: bool = False) -> None:
+    """lorax_sgmv_expand with an optional column window of y.  `transposed`: w_ptr addresses [L, h_out, r]
+    stacks (B^T) instead of the reference's [L, r, h_out]."""
     _check_sgmv(y, x, w_ptr, s_start, s_end, tmp)
     h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
     with torch.cuda.device(x.device):
         rc = lib().lorax_sgmv_expand(
             y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0),
-            x.size(0), x.size(1), h_out, int(y_offset), y.size(1), int(layer_idx), tmp.data_ptr(),
+            x.size(0), x.size(1), h_out, B_HR if transposed else B_RH, int(y_offset), y.size(1), int(layer_idx),
+            tmp.data_ptr(),
             tmp.numel() * tmp.element_size(), _dtype_code(x), _stream(x),
         )
     if rc != 0:

@@ -177,6 +177,9 @@ class RankSegments:
     # address of the B^T stack, 0]. Derived from `indices` and the pointer tables; no counterpart in the
     # reference, whose kernels take one token per thread block.
     plan: Optional[torch.Tensor] = None
+    # prefill: addresses of the transposed B stacks ([L, h_out, r], weights_b_t - the stacks decode uses), one per
+    # segment like lora_b_ptr; the expand kernel for this layout reads each column panel as one contiguous run.
+    lora_b_t_ptr: Optional[torch.Tensor] = None
 
 
 BGMV_PLAN_GROUP = 4
@@ -266,6 +269,10 @@ class BatchLoraWeights(BatchAdapterWeights):
             b_addr = [loras[i].weights_b_t.data_ptr() if i in loras else null for i in seg_adapters]
         lora_a_ptr = torch.tensor(a_addr, dtype=torch.int64, device=device)
         lora_b_ptr = torch.tensor(b_addr, dtype=torch.int64, device=device)
+        lora_b_t_ptr = None
+        if use_sgmv:
+            bt_addr = [loras[i].weights_b_t.data_ptr() if i in loras else null for i in seg_adapters]
+            lora_b_t_ptr = torch.tensor(bt_addr, dtype=torch.int64, device=device)
 
         configs = {seg_adapters[s]: loras[seg_adapters[s]].adapter_config for s in covered}
 
@@ -318,6 +325,7 @@ class BatchLoraWeights(BatchAdapterWeights):
                 segment_ends=ends,
                 indices=token_slots,
                 plan=plan,
+                lora_b_t_ptr=lora_b_t_ptr[segs] if lora_b_t_ptr is not None else None,
             )
 
         return cls(

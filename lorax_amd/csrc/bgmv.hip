@@ -270,7 +270,7 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBat
 // v to the storage type exactly where the two-launch path would store it, and finishes with
 // the expand of its columns.  v never goes to memory and one launch boundary disappears.
 // ---------------------------------------------------------------------------------
-template <typename D, int R, int U, int NBLK, int NT>
+template <typename D, int R, int U, int NBLK, int NT, bool VEC4>
 __device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
                                                const typename D::E* __restrict__ X,
                                                const typename D::E* __restrict__ A,
@@ -293,13 +293,30 @@ __device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
 
   // (1) every B^T vector of the workgroup's column range goes out before the shrink: they do
   // not depend on v, and being cold they are the long pole of the expand.  Clamped, not predicated.
-  auto column = [&](int blk, int u) { return col0 + blk * kBlock + u * kCols + tid / CP; };
+  // VEC4 (every y row 8-byte aligned, h_out a multiple of 4): a lane owns U = 4 adjacent columns, so
+  // the old y of a block is one 8-byte load per token and the new y one 8-byte store, and all of it
+  // is fetched here, ahead of the shrink.  Otherwise lanes take columns kCols apart and y moves
+  // element by element, one block ahead of the arithmetic.
+  typedef E vec4 __attribute__((ext_vector_type(4)));
+  static_assert(!VEC4 || U == 4, "the vector path moves four columns per lane");
+  auto column = [&](int blk, int u) {
+    return VEC4 ? col0 + blk * kBlock + (tid / CP) * U + u : col0 + blk * kBlock + u * kCols + tid / CP;
+  };
   vec8 wv[NBLK][U];
 #pragma unroll
   for (int blk = 0; blk < NBLK; ++blk)
 #pragma unroll
     for (int u = 0; u < U; ++u)
       wv[blk][u] = load8<D>(B + static_cast<int64_t>(min(column(blk, u), h_out - 1)) * R + part * 8);
+  vec4 yq[VEC4 ? NBLK : 1][NT];
+  if constexpr (VEC4) {
+#pragma unroll
+    for (int blk = 0; blk < NBLK; ++blk) {
+      const int cc = min(column(blk, 0), h_out - 4);
+#pragma unroll
+      for (int g = 0; g < NT; ++g) yq[blk][g] = *(const LORAX_GLOBAL vec4*)(yrow[g] + cc);
+    }
+  }
   // the old y of one block (warm: the base projection has just written it)
   auto load_y = [&](int blk, E(&yv)[U][NT]) {
 #pragma unroll
@@ -385,22 +402,50 @@ __device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
       }
     }
   };
-  E ya[U][NT], yb[U][NT];
-  load_y(0, ya);
+  if constexpr (VEC4) {
 #pragma unroll
-  for (int blk = 0; blk < NBLK; blk += 2) {
-    if (col0 + blk * kBlock < col_end) {
-      load_y(blk + 1, yb);
-      __builtin_amdgcn_sched_barrier(0);
-      finish_block(blk, wv[blk], ya);
-      if (blk + 2 < NBLK) load_y(blk + 2, ya);
-      __builtin_amdgcn_sched_barrier(0);
-      finish_block(blk + 1, wv[blk + 1], yb);
+    for (int blk = 0; blk < NBLK; ++blk) {
+      float s[U][NT];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int g = 0; g < NT; ++g) s[u][g] = dot8<D>(wv[blk][u], vv[g], 0.f);
+#pragma unroll
+      for (int m = CP / 2; m >= 1; m >>= 1)
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int g = 0; g < NT; ++g) s[u][g] += __shfl_xor(s[u][g], m, kWave);
+      const int col = column(blk, 0);
+      if (part == 0 && col < col_end) {
+#pragma unroll
+        for (int g = 0; g < NT; ++g) {
+          vec4 out;
+#pragma unroll
+          for (int u = 0; u < U; ++u) out[u] = accumulate<D>(yq[blk][g][u], s[u][g] * scale);
+          *(LORAX_GLOBAL vec4*)(yrow[g] + col) = out;
+        }
+      }
+    }
+  } else {
+    E ya[U][NT], yb[U][NT];
+    load_y(0, ya);
+    if constexpr (NBLK == 1) finish_block(0, wv[0], ya);
+#pragma unroll
+    for (int blk = 0; blk + 1 < NBLK; blk += 2) {
+      if (col0 + blk * kBlock < col_end) {
+        load_y(blk + 1, yb);
+        __builtin_amdgcn_sched_barrier(0);
+        finish_block(blk, wv[blk], ya);
+        if (blk + 2 < NBLK) load_y(blk + 2, ya);
+        __builtin_amdgcn_sched_barrier(0);
+        finish_block(blk + 1, wv[blk + 1], yb);
+      }
     }
   }
 }
 
-template <typename D, int R, int U, int NBLK>
+template <typename D, int R, int U, int NBLK, bool VEC4>
 __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch batch, int h_in,
                                                                  int64_t layer_idx, float scale) {
   using E = typename D::E;
@@ -424,19 +469,19 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch
   const E* X = static_cast<const E*>(P.x);
   switch (n) {
     case 1:
-      bgmv_lora_body<D, R, U, NBLK, 1>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+      bgmv_lora_body<D, R, U, NBLK, 1, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
                                  red, vsh);
       break;
     case 2:
-      bgmv_lora_body<D, R, U, NBLK, 2>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+      bgmv_lora_body<D, R, U, NBLK, 2, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
                                  red, vsh);
       break;
     case 3:
-      bgmv_lora_body<D, R, U, NBLK, 3>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+      bgmv_lora_body<D, R, U, NBLK, 3, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
                                  red, vsh);
       break;
     default:
-      bgmv_lora_body<D, R, U, NBLK, 4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+      bgmv_lora_body<D, R, U, NBLK, 4, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
                                  red, vsh);
       break;
   }
@@ -492,18 +537,42 @@ static hipError_t launch_expand(const BgmvArgs& a, hipStream_t stream) {
   return launch_expand_cp<D, 16>(a, stream);
 }
 
-template <typename D, int R>
-static hipError_t launch_lora_r(const BgmvArgs& a, hipStream_t stream) {
-  // Every column slice of a projection repeats the shrink, so slices are wide: one workgroup
-  // covers 4 expand blocks of 4 columns per lane group (4096 columns at rank 8, 2048 at rank 16)
-  // and holds all their B^T vectors in registers from the start.
+template <typename D, int R, int NBLK>
+static hipError_t launch_lora_blk(const BgmvArgs& a, hipStream_t stream) {
   constexpr int U = 4;
-  constexpr int NBLK = 4;
   constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
   dim3 grid((a.wide_max + cols_per_wg - 1) / cols_per_wg, static_cast<unsigned>(a.grid_rows), a.count);
-  hipLaunchKernelGGL((bgmv_lora_kernel<D, R, U, NBLK>), grid, dim3(kBgmvThreads), 0, stream, a.batch, a.h_in,
-                     a.layer_idx, a.scale);
+  // 8-byte y accesses need every problem's rows 8-byte aligned and no ragged last column group
+  bool vec4 = true;
+  for (int i = 0; i < a.count; ++i) {
+    const BgmvProblem& p = a.batch.p[i];
+    vec4 = vec4 && p.width % 4 == 0 && p.y_stride % 4 == 0 && p.y_offset % 4 == 0 &&
+           reinterpret_cast<uintptr_t>(p.y) % 8 == 0;
+  }
+  if (vec4)
+    hipLaunchKernelGGL((bgmv_lora_kernel<D, R, U, NBLK, true>), grid, dim3(kBgmvThreads), 0, stream, a.batch, a.h_in,
+                       a.layer_idx, a.scale);
+  else
+    hipLaunchKernelGGL((bgmv_lora_kernel<D, R, U, NBLK, false>), grid, dim3(kBgmvThreads), 0, stream, a.batch,
+                       a.h_in, a.layer_idx, a.scale);
   return hipGetLastError();
+}
+
+template <typename D, int R>
+static hipError_t launch_lora_r(const BgmvArgs& a, hipStream_t stream) {
+  // Every column slice of a projection repeats the shrink (its A slab comes from L2 after the first
+  // slice), so slices are as wide as the launch can afford: a workgroup covers NBLK expand blocks of
+  // 4 columns per lane group and holds all their B^T vectors in registers from the start.  A CU
+  // streams only a small share of the chip's bandwidth, so the slices are narrowed until the
+  // launch has workgroups for most of the 256 CUs.
+  constexpr int cols4 = (kBgmvThreads / (R / 8)) * 4 * 4;
+  int64_t wgs4 = 0;
+  for (int i = 0; i < a.count; ++i) wgs4 += a.grid_rows * ((a.batch.p[i].width + cols4 - 1) / cols4);
+  int nblk = wgs4 >= 200 ? 4 : (wgs4 >= 100 ? 2 : 1);
+  if (tuning().bgmv_lora_blocks > 0) nblk = tuning().bgmv_lora_blocks;
+  if (nblk >= 4) return launch_lora_blk<D, R, 4>(a, stream);
+  if (nblk >= 2) return launch_lora_blk<D, R, 2>(a, stream);
+  return launch_lora_blk<D, R, 1>(a, stream);
 }
 
 // y += (x A^T) B^T for planned problems of rank 8 or 16 (a.narrow); a.wide_max is the widest h_out.

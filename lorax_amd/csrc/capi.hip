@@ -95,7 +95,7 @@ int check_common(const void* y, const void* x, const void* w_ptrs, int dtype) {
 const Tuning& tuning() {
   static const Tuning t = {env_int("LORAX_BGMV_LORA_BLOCKS"), env_int("LORAX_BGMV_SHRINK_ROWS"), env_int("LORAX_SHRINK_KSPLIT"),
                            env_int("LORAX_SHRINK_MB"), env_int("LORAX_SHRINK_WAVES"), env_int("LORAX_EXPAND_ROWS"),
-                           env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB")};
+                           env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB"), env_int("LORAX_EXPAND_PANELS")};
   return t;
 }
 
@@ -244,8 +244,9 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
 
 int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
-                      int32_t h_out, int64_t y_offset, int64_t y_stride, int64_t layer_idx,
-                      void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
+                      int32_t h_out, int32_t b_layout, int64_t y_offset, int64_t y_stride,
+                      int64_t layer_idx, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
+  if (b_layout != LORAX_B_RH && b_layout != LORAX_B_HR) return fail(LORAX_EINVAL, "b_layout=%d", b_layout);
   if (num_segments < 0 || num_tokens < 0)
     return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments,
                 (long long)num_tokens);
@@ -277,7 +278,9 @@ int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32
   a.y_stride = y_stride;
   a.layer_idx = layer_idx;
   a.dtype = dtype;
-  const hipError_t e = launch_sgmv_expand(a, static_cast<hipStream_t>(stream));
+  a.a_layout = b_layout;
+  const hipError_t e = b_layout == LORAX_B_HR ? launch_sgmv_expand_t(a, static_cast<hipStream_t>(stream))
+                                              : launch_sgmv_expand(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_expand launch failed: %s", hipGetErrorString(e));
   return LORAX_OK;
 }

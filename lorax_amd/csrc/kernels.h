@@ -57,7 +57,7 @@ struct SgmvArgs {
   int64_t num_tokens;
   int d_in;
   int d_out;
-  int a_layout;  // shrink only
+  int a_layout;  // shrink: LORAX_A_*; expand: LORAX_B_*
   int64_t y_offset;
   int64_t y_stride;
   int64_t layer_idx;
@@ -81,6 +81,7 @@ struct Tuning {
   int shrink_no_rotate;
   int shrink_lds;  // LORAX_SHRINK_LDS: 1 = always take the LDS-staged shrink where it applies, -1 = never
   int shrink_lds_kb;  // LORAX_SHRINK_LDS_KB: LDS budget of the staged shrink's buffers
+  int expand_panels;  // LORAX_EXPAND_PANELS: column panels per wave of the transposed-B expand
 };
 const Tuning& tuning();
 
@@ -88,6 +89,7 @@ hipError_t launch_bgmv(const BgmvArgs& a, hipStream_t stream);
 hipError_t launch_bgmv_lora(const BgmvArgs& a, hipStream_t stream);
 hipError_t launch_sgmv_shrink(const SgmvArgs& a, hipStream_t stream);
 hipError_t launch_sgmv_expand(const SgmvArgs& a, hipStream_t stream);
+hipError_t launch_sgmv_expand_t(const SgmvArgs& a, hipStream_t stream);  // B stacks stored as [L, h_out, r]
 // LDS-staged shrink (sgmv_shrink_lds.hip): [L, r, h_in] layout, h_in a multiple of 128.
 bool sgmv_shrink_lds_applies(const SgmvArgs& a);
 hipError_t launch_sgmv_shrink_lds(const SgmvArgs& a, hipStream_t stream);

@@ -93,7 +93,13 @@ class LoraLinear(nn.Module):
                 )
                 if tensor_parallel:
                     v = self.collect_lora_a(v)
-                if sliced:
+                if rs.lora_b_t_ptr is not None:
+                    # transposed B stacks (resident for decode anyway): the faster expand
+                    lora_b_sgmv_cutlass_slice(
+                        result, v, rs.tmp_expand, rs.lora_b_t_ptr, rs.segment_starts, rs.segment_ends,
+                        self.layer_id, start, end - start, transposed=True,
+                    )
+                elif sliced:
                     lora_b_sgmv_cutlass_slice(
                         result, v, rs.tmp_expand, rs.lora_b_ptr, rs.segment_starts, rs.segment_ends,
                         self.layer_id, start, end - start,

@@ -198,9 +198,12 @@ def add_lora_b_bgmv_slice(y, v, wb_T_all, indicies, layer_idx, y_offset: int, y_
     _native_module().bgmv(y, v, wb_T_all, indicies, layer_idx, 1.0, y_offset, y_slice_size)
 
 
-def lora_b_sgmv_cutlass_slice(y, v, tmp, wb_ptr, s_start, s_end, layer_idx, y_offset: int, y_slice_size: int):
-    """As lora_b_sgmv_cutlass, writing columns [y_offset, y_offset + y_slice_size) of a wider y."""
-    _native_module().sgmv_expand(y, v, wb_ptr, s_start, s_end, tmp, layer_idx, y_offset, y_slice_size)
+def lora_b_sgmv_cutlass_slice(y, v, tmp, wb_ptr, s_start, s_end, layer_idx, y_offset: int, y_slice_size: int,
+                              transposed: bool = False):
+    """As lora_b_sgmv_cutlass, writing columns [y_offset, y_offset + y_slice_size) of a wider y.  With
+    `transposed`, wb_ptr addresses the [L, h_out, r] stacks of the decode path (weights_b_t) - same result,
+    faster kernel."""
+    _native_module().sgmv_expand(y, v, wb_ptr, s_start, s_end, tmp, layer_idx, y_offset, y_slice_size, transposed)
 
 
 def segmented_matmul(

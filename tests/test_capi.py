@@ -76,12 +76,14 @@ def test_sgmv_shrink_validation():
 
 def test_sgmv_expand_validation():
     f = _native.lib().lorax_sgmv_expand
-    assert f(P, P, P, P, P, 2, 16, 16, 4096, 0, 4096, 0, P, 121, 1, None) == ETMPSIZE
-    assert f(P, P, P, P, P, 0, 16, 16, 4096, 0, 4096, 0, None, 0, 1, None) == OK
-    for r, h in [(4, 4096), (136, 4096), (16, 4100)]:
-        assert f(P, P, P, P, P, 2, 16, r, h, 0, h, 0, P, 120, 1, None) == ENOKERNEL, (r, h)
-    assert f(P, P, P, P, P, 2, 16, 16, 4096, 4, 8192, 0, P, 120, 1, None) == EINVAL  # unaligned window
-    assert f(P, P, P, P, P, 2, 16, 16, 4096, 4096, 4096, 0, P, 120, 1, None) == EINVAL  # window too wide
+    for layout in (_native.B_RH, _native.B_HR):
+        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 0, 4096, 0, P, 121, 1, None) == ETMPSIZE
+        assert f(P, P, P, P, P, 0, 16, 16, 4096, layout, 0, 4096, 0, None, 0, 1, None) == OK
+        for r, h in [(4, 4096), (136, 4096), (16, 4100)]:
+            assert f(P, P, P, P, P, 2, 16, r, h, layout, 0, h, 0, P, 120, 1, None) == ENOKERNEL, (r, h)
+        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 4, 8192, 0, P, 120, 1, None) == EINVAL  # unaligned window
+        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 4096, 4096, 0, P, 120, 1, None) == EINVAL  # too wide
+    assert f(P, P, P, P, P, 2, 16, 16, 4096, 2, 0, 4096, 0, P, 120, 1, None) == EINVAL  # unknown layout
 
 
 def test_python_binding_rejects_cpu_tensors():

@@ -158,6 +158,55 @@ def test_sgmv_shrink_tile_variants(r, h_in, lens):
     assert torch.count_nonzero(v.cpu()[~covered]) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("r", [8, 16, 24, 32, 64, 96, 128])
+@pytest.mark.parametrize("h_out,lens,window", [
+    (4096, [16, 16, 16, 16], None),
+    (2048, [1, 0, 3, 17, 1, 64, 5, 0, 130], None),
+    (1160, [300, 2, 31, 257], None),             # 18 panels of 64 columns and one of 8
+    (1024, [70, 1, 1, 600], (512, 384)),         # a column window of a wider y
+    (8, [5, 40], None),
+])
+def test_sgmv_expand_transposed_b(dtype, r, h_out, lens, window):
+    """lorax_sgmv_expand with b_layout = LORAX_B_HR ([L, h_out, r] stacks) against the oracle on the
+    reference layout, and against the kernel for the reference layout."""
+    print(f"case dtype={dtype} r={r} h_out={h_out} lens={lens} window={window}", flush=True)
+    gen = torch.Generator().manual_seed(r * 11 + h_out)
+    layer = 1
+    T, _, y0, _, wb, starts, ends = _ragged_case(dtype, r, 64, h_out, lens, gen)
+    v = randn((T, r), 1.0, gen, dtype, DEV)
+    off, width = window if window is not None else (0, h_out)
+    if window is not None:
+        wb = [w[:, :, :width].contiguous() if w is not None else None for w in wb]
+    wbt = [w.transpose(1, 2).contiguous() if w is not None else None for w in wb]
+    s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
+    tmp = sgmv.get_tmp_expand_size(len(starts))
+    tmp = torch.empty((tmp,), dtype=torch.uint8, device=DEV)
+    y_t, y_n = y0.clone(), y0.clone()
+    sgmv.lora_b_sgmv_cutlass_slice(y_t, v, tmp, ptr_table(wbt, DEV), s_start, s_end, layer, off, width, transposed=True)
+    sgmv.lora_b_sgmv_cutlass_slice(y_n, v, tmp, ptr_table(wb, DEV), s_start, s_end, layer, off, width)
+    torch.cuda.synchronize()
+    y_ref = y0.cpu().clone()
+    for i, (s, e) in enumerate(zip(starts, ends)):
+        if e > s:
+            delta = v.cpu()[s:e] @ wb[i][layer].cpu()
+            y_ref[s:e, off:off + width] = y_ref[s:e, off:off + width] + delta
+    assert_close(y_t, y_ref, "transposed-B expand", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
+    # Segments of more than 4 rows run the same MFMA arithmetic in the same order for both layouts (the
+    # reference-layout kernel sums shorter ones on the vector ALU).
+    long_rows = torch.zeros(T, dtype=torch.bool)
+    for s, e in zip(starts, ends):
+        if e - s > 4:
+            long_rows[s:e] = True
+    assert torch.equal(y_t.cpu()[long_rows], y_n.cpu()[long_rows])
+    assert_close(y_n, y_ref, "reference-layout expand", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
+    outside = torch.ones_like(y0, dtype=torch.bool).cpu()
+    for s, e in zip(starts, ends):
+        outside[s:e, off:off + width] = False
+    assert torch.equal(y_t.cpu()[outside], y0.cpu()[outside])
+
+
 @pytest.mark.parametrize("r", [48, 80, 96, 112])
 def test_sgmv_other_multiples_of_16(r):
     """pad_to_min_rank can produce these ranks (punica.py:57-65); the reference's shrink has no
