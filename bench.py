@@ -102,15 +102,17 @@ class Plan:
                     self._add_bgmv_reference(x, y, off, size, group.h_in, r, rd)
                 else:
                     decode[r].append((rd, off, size))
-            for r, rank_jobs in decode.items():
-                single = []
-                if self.use_plan and self.fuse_small_ranks:
-                    single = [j for j in rank_jobs if _native.bgmv_lora_fits(r, group.h_in, j[2])]
-                    rank_jobs = [j for j in rank_jobs if not any(j is s for s in single)]
-                for i in range(0, len(single), 4):
-                    self._add_bgmv_fused(x, y, group.h_in, r, single[i:i + 4], single_launch=True)
-                for i in range(0, len(rank_jobs), 4):
-                    self._add_bgmv_fused(x, y, group.h_in, r, rank_jobs[i:i + 4], single_launch=False)
+            all_jobs = [(r, rd, off, size) for r, rank_jobs in decode.items() for rd, off, size in rank_jobs]
+            all_fused = bool(all_jobs) and self.use_plan and self.fuse_small_ranks and all(
+                _native.bgmv_lora_fits(r, group.h_in, size) for r, _, _, size in all_jobs)
+            if all_fused:
+                for r, rank_jobs in decode.items():
+                    for i in range(0, len(rank_jobs), _native.MAX_FUSED_BGMV_PROBLEMS):
+                        self._add_bgmv_fused(x, y, group.h_in, [(r,) + j for j in rank_jobs[i:i + 4]], True)
+            else:
+                step = _native.MAX_BGMV_PROBLEMS
+                for i in range(0, len(all_jobs), step):
+                    self._add_bgmv_fused(x, y, group.h_in, all_jobs[i:i + step], False)
 
     @staticmethod
     def _bgmv_counts(rd):
@@ -169,34 +171,37 @@ class Plan:
                            lambda layer: sgmv.add_lora_b_bgmv_slice(y, v, b_ptr, idx, layer, off, size),
                            rows * r * e + uniq * r * size * e + 2 * rows * size * e, 2 * rows * r * size))
 
-    def _add_bgmv_fused(self, x, y, h_in, r, jobs, single_launch):
+    def _add_bgmv_fused(self, x, y, h_in, jobs, single_launch):
+        """jobs: (rank, rank_segments, column offset, width); one rank for the single launch, any mix otherwise."""
         import torch
 
         from lorax_amd import _native
 
         e = 2
-        vs = torch.zeros((len(jobs), x.size(0), r), dtype=x.dtype, device=x.device).unbind(0)
-        shrink_problems = [(v, x, rd.lora_a_ptr, rd.indices, 0, None) for v, (rd, _, _) in zip(vs, jobs)]
-        expand_problems = [(y, v, rd.lora_b_ptr, rd.indices, off, size) for v, (rd, off, size) in zip(vs, jobs)]
-        counts = [self._bgmv_counts(rd) for rd, _, _ in jobs]
-        any_routed = torch.stack([rd.indices >= 0 for rd, _, _ in jobs]).any(0)
+        vs = [torch.zeros((x.size(0), r), dtype=x.dtype, device=x.device) for r, _, _, _ in jobs]
+        shrink_problems = [(v, x, rd.lora_a_ptr, rd.indices, 0, None) for v, (_, rd, _, _) in zip(vs, jobs)]
+        expand_problems = [(y, v, rd.lora_b_ptr, rd.indices, off, size) for v, (_, rd, off, size) in zip(vs, jobs)]
+        counts = [self._bgmv_counts(rd) for _, rd, _, _ in jobs]
+        any_routed = torch.stack([rd.indices >= 0 for _, rd, _, _ in jobs]).any(0)
         x_rows = int(any_routed.sum().item())  # the shared input is read once per launch
-        shrink_bytes = x_rows * h_in * e + sum(u * r * h_in * e + n * r * e for n, u in counts)
+        shrink_bytes = x_rows * h_in * e + sum(u * r * h_in * e + n * r * e for (n, u), (r, _, _, _) in zip(counts, jobs))
         expand_bytes = sum(n * r * e + u * r * size * e + 2 * n * size * e
-                           for (n, u), (_, _, size) in zip(counts, jobs))
-        plans = [rd.plan for rd, _, _ in jobs] if self.use_plan else None
+                           for (n, u), (r, _, _, size) in zip(counts, jobs))
+        plans = [rd.plan for _, rd, _, _ in jobs] if self.use_plan else None
         if single_launch:
-            lora_problems = [(y, x, rd.plan, off, size) for rd, off, size in jobs]
+            r = jobs[0][0]
+            lora_problems = [(y, x, rd.plan, off, size) for _, rd, off, size in jobs]
             # v stays on chip: its write by the shrink and read by the expand are not memory traffic
             v_bytes = sum(2 * n * r * e for n, _ in counts)
             self.calls.append(("bgmv_lora", lambda layer: _native.bgmv_lora_multi(lora_problems, r, layer),
                                shrink_bytes + expand_bytes - v_bytes,
-                               sum(2 * n * r * (h_in + size) for (n, _), (_, _, size) in zip(counts, jobs))))
+                               sum(2 * n * r * (h_in + size) for (n, _), (_, _, _, size) in zip(counts, jobs))))
             return
         self.calls.append(("bgmv_shrink", lambda layer: _native.bgmv_multi(shrink_problems, layer, 1.0, False, plans),
-                           shrink_bytes, sum(2 * n * r * h_in for n, _ in counts)))
+                           shrink_bytes, sum(2 * n * r * h_in for (n, _), (r, _, _, _) in zip(counts, jobs))))
         self.calls.append(("bgmv_expand", lambda layer: _native.bgmv_multi(expand_problems, layer, 1.0, True, plans),
-                           expand_bytes, sum(2 * n * r * size for (n, _), (_, _, size) in zip(counts, jobs))))
+                           expand_bytes,
+                           sum(2 * n * r * size for (n, _), (r, _, _, size) in zip(counts, jobs))))
 
     def issue(self, layers, kinds=None):
         n = 0

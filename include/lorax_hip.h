@@ -86,10 +86,13 @@ int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* ind
  * exists because a decode-size BGMV is shorter than a launch, so the projections that share an
  * input (q/k/v, gate/up) are better issued together.
  *
- * `problems` is a HOST array of `num_problems` (<= 4) descriptors; the pointers inside are
- * device pointers.  All problems share num_tokens, h_in, layer_idx, scale, dtype, the direction
- * (h_in < h_out means expand) and the LoRA rank; expand problems may differ in h_out.  Each
- * problem is computed exactly as by lorax_bgmv.  accumulate = 0 (shrink launches only) stores
+ * `problems` is a HOST array of `num_problems` (<= 16) descriptors; the pointers inside are
+ * device pointers.  All problems share num_tokens, layer_idx, scale, dtype and the direction
+ * (h_in < h_out means expand).  Shrink problems share h_in and may differ in rank (their h_out);
+ * expand problems may differ in rank (the problem's own h_in field) and in h_out - so the rank
+ * groups of a multi-rank batch (lorax_server/adapters/lora.py:339-348, one kernel call per rank
+ * in the reference) go out in ONE shrink launch and ONE expand launch.  Each problem is computed
+ * exactly as by lorax_bgmv.  accumulate = 0 (shrink launches only) stores
  * dtype(sum) instead of adding it, so the caller need not zero v first; rows of tokens whose
  * index is negative are not written in either mode.
  *
@@ -114,6 +117,7 @@ typedef struct lorax_bgmv_problem {
   int32_t h_out;
   const int64_t* plan;    /* optional routing plan (see above), else NULL          */
   int32_t num_groups;     /* records in plan                                       */
+  int32_t h_in;           /* this problem's input width; 0 = the call's h_in       */
 } lorax_bgmv_problem_t;
 
 int lorax_bgmv_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems, int64_t num_tokens,

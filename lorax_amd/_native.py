@@ -38,10 +38,12 @@ class BgmvProblem(ctypes.Structure):
         ("h_out", _c.c_int32),
         ("plan", _c.c_void_p),
         ("num_groups", _c.c_int32),
+        ("h_in", _c.c_int32),
     ]
 
 
-MAX_BGMV_PROBLEMS = 4
+MAX_BGMV_PROBLEMS = 16
+MAX_FUSED_BGMV_PROBLEMS = 4
 
 _SIGNATURES = {
     "lorax_bgmv": (
@@ -209,8 +211,10 @@ PLAN_RECORD_WORDS = 8
 
 
 def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> None:
-    """lorax_bgmv_multi: `problems` is a list of up to 4 tuples (y, x, w_ptr, indicies, y_offset, y_slice_size)
-    that share x.shape, the direction and the rank; y_slice_size None means the whole width of y.
+    """lorax_bgmv_multi: `problems` is a list of up to 16 tuples (y, x, w_ptr, indicies, y_offset, y_slice_size)
+    that share the token count and the direction; shrink problems share x.shape and may differ in rank
+    (y's width), expand problems may differ in rank (x's width) and output width.  y_slice_size None means
+    the whole width of y.
     `plans`, if given, holds one routing plan per problem: an int64 device tensor [num_groups, 8]."""
     if not 1 <= len(problems) <= MAX_BGMV_PROBLEMS:
         raise RuntimeError(f"between 1 and {MAX_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
@@ -224,8 +228,8 @@ def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> N
         _check_same(y, x, w_ptr, indicies)
         if w_ptr.dtype != torch.int64 or indicies.dtype != torch.int64:
             raise RuntimeError("w_ptr and indicies must be int64 tensors")
-        if x.shape != x0.shape or x.dtype != x0.dtype or x.device != x0.device:
-            raise RuntimeError("all problems of one launch must have inputs of one shape, dtype and device")
+        if x.size(0) != x0.size(0) or x.dtype != x0.dtype or x.device != x0.device:
+            raise RuntimeError("all problems of one launch must have inputs of one row count, dtype and device")
         if indicies.size(0) != x.size(0) or y.size(0) != x.size(0):
             raise RuntimeError(
                 f"CHECK_EQ(indicies.size(0), x.size(0)) / CHECK_EQ(y.size(0), x.size(0)) failed. "
@@ -242,7 +246,7 @@ def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> N
             if num_groups == 0:
                 plan_ptr = x.data_ptr()  # an empty plan has no storage; any non-null address will do
         arr[i] = BgmvProblem(y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), indicies.data_ptr(), int(y_offset),
-                             y.size(1), h_out, plan_ptr, num_groups)
+                             y.size(1), h_out, plan_ptr, num_groups, x.size(1))
     with torch.cuda.device(x0.device):
         rc = lib().lorax_bgmv_multi(arr, len(problems), x0.size(0), x0.size(1), int(layer_idx), float(scale),
                                     1 if accumulate else 0, _dtype_code(x0), _stream(x0))
@@ -266,8 +270,8 @@ def bgmv_lora_fits(rank: int, h_in: int, h_out: int) -> bool:
 def bgmv_lora_multi(problems, rank, layer_idx, scale=1.0) -> None:
     """lorax_bgmv_lora_multi: `problems` is a list of up to 4 tuples (y, x, plan, y_offset, y_slice_size) that
     share x.shape; y[:, window] += (x @ A^T) @ B^T per planned token chunk, rank 8 or 16."""
-    if not 1 <= len(problems) <= MAX_BGMV_PROBLEMS:
-        raise RuntimeError(f"between 1 and {MAX_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
+    if not 1 <= len(problems) <= MAX_FUSED_BGMV_PROBLEMS:
+        raise RuntimeError(f"between 1 and {MAX_FUSED_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
     arr = (BgmvProblem * len(problems))()
     x0 = problems[0][1]
     for i, (y, x, plan, y_offset, y_slice_size) in enumerate(problems):

@@ -110,6 +110,21 @@ __device__ __forceinline__ void bgmv_shrink_body(typename D::E* __restrict__ Y,
   }
 }
 
+// Problem, token chunk and row block / column slice of this workgroup (see BgmvBatch).  Wave-uniform.
+struct BatchSlot {
+  int problem, chunk, sub;
+};
+__device__ __forceinline__ BatchSlot batch_slot(const BgmvBatch& batch, int count) {
+  const int v = static_cast<int>(xcd_virtual_id());
+  int p = 0;
+  while (p + 1 < count && v >= batch.run_end[p]) ++p;  // first problem of the run that holds v
+  const int rem = v - batch.base[p];
+  const int run_subs = batch.run_subs[p];
+  const int chunk = rem / run_subs, s = rem % run_subs;
+  while (p + 1 < count && s >= batch.sub_hi[p]) ++p;
+  return BatchSlot{p, chunk, s - batch.sub_lo[p]};
+}
+
 // Resolves the token chunk of workgroup row `row` and the address of its adapter's stack.
 // With a routing plan (built once per batch next to the index tables) this is one 64-byte
 // record: [ntok, tok0..tok3, address of the A stack, address of the B^T stack, reserved];
@@ -135,17 +150,18 @@ __device__ __forceinline__ int resolve_chunk(const BgmvProblem& P, int num_token
 
 template <typename D, int RS>
 __global__ __launch_bounds__(kBgmvThreads) void bgmv_shrink_kernel(
-    const BgmvBatch batch, int num_tokens, int h_in, int r, int64_t layer_idx, float scale,
+    const BgmvBatch batch, int count, int num_tokens, int h_in, int64_t layer_idx, float scale,
     int accumulate_into_y) {
   __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<RS * kGroup>::value];
   using E = typename D::E;
-  const VirtualBlock vb = xcd_virtual_block();
-  const BgmvProblem& P = batch.p[vb.z];
+  const BatchSlot slot = batch_slot(batch, count);
+  const BgmvProblem& P = batch.p[slot.problem];
+  const int r = P.narrow;
+  const int row0 = slot.sub * RS;
   int toks[kGroup];
   int64_t stack_addr;
-  const int n = resolve_chunk(P, num_tokens, false, vb.y, toks, stack_addr);
+  const int n = resolve_chunk(P, num_tokens, false, slot.chunk, toks, stack_addr);
   if (n == 0) return;
-  const int row0 = vb.x * RS;
   const E* A = reinterpret_cast<const E*>(stack_addr) + (layer_idx * r + row0) * static_cast<int64_t>(h_in);
   E* Y = static_cast<E*>(P.y);
   const E* X = static_cast<const E*>(P.x);
@@ -229,18 +245,15 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
 }
 
 template <typename D, int CP, int U>
-__global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBatch batch,
-                                                                   int num_tokens, int r,
-                                                                   int64_t layer_idx, float scale) {
+__device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const BatchSlot& slot, int num_tokens,
+                                                    int64_t layer_idx, float scale) {
   using E = typename D::E;
-  const VirtualBlock vb = xcd_virtual_block();
-  const BgmvProblem& P = batch.p[vb.z];
   const int h_out = P.width;
-  const int col0 = vb.x * (kBgmvThreads / CP) * U;
-  if (col0 >= h_out) return;  // problems of one batch may differ in width
+  const int r = P.narrow;
+  const int col0 = slot.sub * (kBgmvThreads / CP) * U;
   int toks[kGroup];
   int64_t stack_addr;
-  const int n = resolve_chunk(P, num_tokens, true, vb.y, toks, stack_addr);
+  const int n = resolve_chunk(P, num_tokens, true, slot.chunk, toks, stack_addr);
   if (n == 0) return;
   const E* B = reinterpret_cast<const E*>(stack_addr) + layer_idx * h_out * static_cast<int64_t>(r);
   E* Y = static_cast<E*>(P.y);
@@ -257,6 +270,37 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBat
       break;
     default:
       bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
+      break;
+  }
+}
+
+// Lanes per column of a rank: the power of two >= r / 8.
+__host__ __device__ __forceinline__ int expand_lanes_per_column(int r) {
+  const int chunks = r / 8;
+  return chunks <= 1 ? 1 : (chunks <= 2 ? 2 : (chunks <= 4 ? 4 : (chunks <= 8 ? 8 : 16)));
+}
+
+// One launch serves problems of different ranks: the workgroup picks the body for its problem's rank.
+template <typename D, int U>
+__global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBatch batch, int count,
+                                                                   int num_tokens, int64_t layer_idx, float scale) {
+  const BatchSlot vb = batch_slot(batch, count);
+  const BgmvProblem& P = batch.p[vb.problem];
+  switch (expand_lanes_per_column(P.narrow)) {
+    case 1:
+      bgmv_expand_problem<D, 1, U>(P, vb, num_tokens, layer_idx, scale);
+      break;
+    case 2:
+      bgmv_expand_problem<D, 2, U>(P, vb, num_tokens, layer_idx, scale);
+      break;
+    case 4:
+      bgmv_expand_problem<D, 4, U>(P, vb, num_tokens, layer_idx, scale);
+      break;
+    case 8:
+      bgmv_expand_problem<D, 8, U>(P, vb, num_tokens, layer_idx, scale);
+      break;
+    default:
+      bgmv_expand_problem<D, 16, U>(P, vb, num_tokens, layer_idx, scale);
       break;
   }
 }
@@ -490,11 +534,42 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch
 // ---------------------------------------------------------------------------------
 // Host-side launchers
 // ---------------------------------------------------------------------------------
+// Fills the workgroup numbering of a batch (see BgmvBatch); subs_of(problem) is the number of row
+// blocks / column slices of one token chunk.  Returns the number of workgroups.
+template <typename SubsOf>
+static int64_t number_workgroups(BgmvArgs& a, SubsOf subs_of) {
+  auto chunks_of = [&](int i) {
+    return a.batch.p[i].plan != nullptr ? static_cast<int64_t>(a.batch.p[i].num_groups) : a.num_tokens;
+  };
+  int64_t total = 0;
+  for (int first = 0; first < a.count;) {
+    int last = first;
+    while (!tuning().bgmv_no_runs && last + 1 < a.count && chunks_of(last + 1) == chunks_of(first)) ++last;
+    int run_subs = 0;
+    for (int i = first; i <= last; ++i) {
+      a.batch.sub_lo[i] = run_subs;
+      run_subs += subs_of(a.batch.p[i]);
+      a.batch.sub_hi[i] = run_subs;
+    }
+    const int64_t end = total + chunks_of(first) * run_subs;
+    for (int i = first; i <= last; ++i) {
+      a.batch.base[i] = static_cast<int>(total < INT32_MAX ? total : INT32_MAX);
+      a.batch.run_subs[i] = run_subs > 0 ? run_subs : 1;
+      a.batch.run_end[i] = static_cast<int>(end < INT32_MAX ? end : INT32_MAX);
+    }
+    total = end;
+    first = last + 1;
+  }
+  return total;
+}
+
 template <typename D, int RS>
-static hipError_t launch_shrink_rs(const BgmvArgs& a, hipStream_t stream) {
-  dim3 grid(a.narrow / RS, static_cast<unsigned>(a.grid_rows), a.count);
-  hipLaunchKernelGGL((bgmv_shrink_kernel<D, RS>), grid, dim3(kBgmvThreads), 0, stream, a.batch,
-                     static_cast<int>(a.num_tokens), a.wide_max, a.narrow, a.layer_idx, a.scale,
+static hipError_t launch_shrink_rs(BgmvArgs a, hipStream_t stream) {
+  const int64_t total = number_workgroups(a, [](const BgmvProblem& p) { return p.narrow / RS; });
+  if (total == 0) return hipSuccess;
+  if (total >= INT32_MAX) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((bgmv_shrink_kernel<D, RS>), dim3(static_cast<unsigned>(total)), dim3(kBgmvThreads), 0, stream,
+                     a.batch, a.count, static_cast<int>(a.num_tokens), a.wide_max, a.layer_idx, a.scale,
                      a.accumulate);
   return hipGetLastError();
 }
@@ -503,7 +578,7 @@ template <typename D>
 static hipError_t launch_shrink(const BgmvArgs& a, hipStream_t stream) {
   // Rows per workgroup: 8 when the grid is large enough to fill 256 CUs several times
   // over, fewer rows (more workgroups) for small batches.
-  const int64_t wgs8 = a.work_rows * (a.narrow / 8) * a.count;
+  const int64_t wgs8 = a.work_rows * (a.narrow_sum / 8);
   int rs = wgs8 >= 2048 ? 8 : (wgs8 >= 512 ? 4 : 2);
   if (tuning().bgmv_shrink_rows > 0) rs = tuning().bgmv_shrink_rows;
   switch (rs) {
@@ -516,25 +591,31 @@ static hipError_t launch_shrink(const BgmvArgs& a, hipStream_t stream) {
   }
 }
 
-template <typename D, int CP>
-static hipError_t launch_expand_cp(const BgmvArgs& a, hipStream_t stream) {
-  constexpr int U = 4;
-  constexpr int cols_per_wg = (kBgmvThreads / CP) * U;
-  dim3 grid((a.wide_max + cols_per_wg - 1) / cols_per_wg, static_cast<unsigned>(a.grid_rows),
-            a.count);
-  hipLaunchKernelGGL((bgmv_expand_kernel<D, CP, U>), grid, dim3(kBgmvThreads), 0, stream, a.batch,
-                     static_cast<int>(a.num_tokens), a.narrow, a.layer_idx, a.scale);
+template <typename D, int U>
+static hipError_t launch_expand_u(BgmvArgs a, hipStream_t stream) {
+  const int64_t total = number_workgroups(a, [](const BgmvProblem& p) {
+    const int cols_per_wg = (kBgmvThreads / expand_lanes_per_column(p.narrow)) * U;
+    return (p.width + cols_per_wg - 1) / cols_per_wg;
+  });
+  if (total == 0) return hipSuccess;
+  if (total >= INT32_MAX) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((bgmv_expand_kernel<D, U>), dim3(static_cast<unsigned>(total)), dim3(kBgmvThreads), 0, stream,
+                     a.batch, a.count, static_cast<int>(a.num_tokens), a.layer_idx, a.scale);
   return hipGetLastError();
 }
 
 template <typename D>
 static hipError_t launch_expand(const BgmvArgs& a, hipStream_t stream) {
-  const int chunks = a.narrow / 8;
-  if (chunks <= 1) return launch_expand_cp<D, 1>(a, stream);
-  if (chunks <= 2) return launch_expand_cp<D, 2>(a, stream);
-  if (chunks <= 4) return launch_expand_cp<D, 4>(a, stream);
-  if (chunks <= 8) return launch_expand_cp<D, 8>(a, stream);
-  return launch_expand_cp<D, 16>(a, stream);
+  // Columns per lane group.  Narrow slices win: the launch is a long list of independent small
+  // workgroups and the CUs overlap their routing-record and weight round trips across workgroups.
+  int64_t bytes = 0;
+  for (int i = 0; i < a.count; ++i)
+    bytes += a.work_rows * a.batch.p[i].width * static_cast<int64_t>(a.batch.p[i].narrow) * 2;
+  int u = bytes >= (32ll << 20) ? 4 : 2;
+  if (tuning().bgmv_expand_cols > 0) u = tuning().bgmv_expand_cols;
+  if (u >= 8) return launch_expand_u<D, 8>(a, stream);
+  if (u <= 2) return launch_expand_u<D, 2>(a, stream);
+  return launch_expand_u<D, 4>(a, stream);
 }
 
 template <typename D, int R, int NBLK>

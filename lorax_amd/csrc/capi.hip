@@ -95,7 +95,7 @@ int check_common(const void* y, const void* x, const void* w_ptrs, int dtype) {
 const Tuning& tuning() {
   static const Tuning t = {env_int("LORAX_BGMV_LORA_BLOCKS"), env_int("LORAX_BGMV_SHRINK_ROWS"), env_int("LORAX_SHRINK_KSPLIT"),
                            env_int("LORAX_SHRINK_MB"), env_int("LORAX_SHRINK_WAVES"), env_int("LORAX_EXPAND_ROWS"),
-                           env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB"), env_int("LORAX_EXPAND_PANELS")};
+                           env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB"), env_int("LORAX_BGMV_EXPAND_COLS"), env_int("LORAX_EXPAND_PANELS"), env_int("LORAX_BGMV_NO_RUNS")};
   return t;
 }
 
@@ -105,8 +105,9 @@ using namespace lorax;
 
 namespace {
 
-// Validates one batch of BGMV problems that share num_tokens, h_in, direction and layer and
-// launches it.  h_out[i] is problem i's output width.
+// Validates one batch of BGMV problems that share num_tokens, direction and layer and launches it.
+// Problem i maps its own h_in (the call's h_in where the field is 0) to its own h_out; shrink problems
+// share h_in and may differ in rank (h_out), expand problems may differ in rank (h_in) and width.
 int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_tokens, int32_t h_in,
                int64_t layer_idx, float scale, int32_t accumulate, int32_t dtype, void* stream) {
   if (count < 0 || count > kMaxBgmvProblems)
@@ -117,8 +118,7 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
   if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
   BgmvArgs a{};
   a.count = count;
-  a.expand = h_in < problems[0].h_out;  // bgmv_impl.cuh:204
-  a.narrow = a.expand ? h_in : problems[0].h_out;
+  a.expand = (problems[0].h_in > 0 ? problems[0].h_in : h_in) < problems[0].h_out;  // bgmv_impl.cuh:204
   a.wide_max = a.expand ? 0 : h_in;
   a.num_tokens = num_tokens;
   a.layer_idx = layer_idx;
@@ -140,21 +140,27 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
       if (q.indices == nullptr) return fail(LORAX_EINVAL, "null pointer argument (indices)");
     }
     const int h_out = q.h_out;
-    const bool expand = h_in < h_out;
-    const int narrow = expand ? h_in : h_out;
-    const int wide = expand ? h_out : h_in;
+    const int q_in = q.h_in > 0 ? q.h_in : h_in;
+    const bool expand = q_in < h_out;
+    const int narrow = expand ? q_in : h_out;
+    const int wide = expand ? h_out : q_in;
     // punica_ops.cc:310 (dims < 65536) and bgmv_config.h:12-86 (narrow side 8..128).
-    if (h_in <= 0 || h_out <= 0 || h_in >= 65536 || h_out >= 65536 || narrow % 8 != 0 ||
+    if (q_in <= 0 || h_out <= 0 || q_in >= 65536 || h_out >= 65536 || narrow % 8 != 0 ||
         narrow > kMaxRank || wide % 8 != 0)
-      return fail(LORAX_ENOKERNEL, "No suitable kernel. h_in=%d h_out=%d dtype=%d", h_in, h_out, dtype);
-    if (expand != a.expand || narrow != a.narrow)
-      return fail(LORAX_EINVAL, "problems of one launch must share direction and rank (problem %d: h_out=%d)",
-                  i, h_out);
+      return fail(LORAX_ENOKERNEL, "No suitable kernel. h_in=%d h_out=%d dtype=%d", q_in, h_out, dtype);
+    if (expand != a.expand)
+      return fail(LORAX_EINVAL, "problems of one launch must share the direction (problem %d: h_in=%d h_out=%d)", i,
+                  q_in, h_out);
+    if (!expand && q_in != h_in)
+      return fail(LORAX_EINVAL, "shrink problems of one launch share h_in=%d (problem %d: h_in=%d)", h_in, i, q_in);
     if (q.y_offset < 0 || q.y_stride < q.y_offset + h_out)
       return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld do not hold h_out=%d columns",
                   (long long)q.y_offset, (long long)q.y_stride, h_out);
     if (a.expand && h_out > a.wide_max) a.wide_max = h_out;
-    a.batch.p[i] = BgmvProblem{q.y, q.x, q.w_ptrs, q.indices, q.y_offset, q.y_stride, h_out, q.plan, q.num_groups};
+    if (narrow > a.narrow) a.narrow = narrow;
+    a.narrow_sum += narrow;
+    a.batch.p[i] =
+        BgmvProblem{q.y, q.x, q.w_ptrs, q.indices, q.y_offset, q.y_stride, wide, narrow, q.plan, q.num_groups};
   }
   if (!planned) a.grid_rows = num_tokens;
   a.work_rows = planned ? a.grid_rows : (num_tokens + 1) / 2;
@@ -178,7 +184,7 @@ int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* ind
                int64_t num_tokens, int32_t h_in, int32_t h_out, int64_t y_offset,
                int64_t y_stride, int64_t layer_idx, float scale, int32_t dtype, void* stream) {
   if (num_tokens == 0) return LORAX_OK;
-  const lorax_bgmv_problem_t one{y, x, w_ptrs, indices, y_offset, y_stride, h_out, nullptr, 0};
+  const lorax_bgmv_problem_t one{y, x, w_ptrs, indices, y_offset, y_stride, h_out, nullptr, 0, 0};
   return bgmv_batch(&one, 1, num_tokens, h_in, layer_idx, scale, 1, dtype, stream);
 }
 
@@ -288,8 +294,8 @@ int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32
 int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems, int64_t num_tokens,
                           int32_t h_in, int32_t r, int64_t layer_idx, float scale, int32_t dtype,
                           void* stream) {
-  if (num_problems < 0 || num_problems > kMaxBgmvProblems)
-    return fail(LORAX_EINVAL, "num_problems=%d (at most %d per launch)", num_problems, kMaxBgmvProblems);
+  if (num_problems < 0 || num_problems > kMaxFusedBgmvProblems)
+    return fail(LORAX_EINVAL, "num_problems=%d (at most %d per launch)", num_problems, kMaxFusedBgmvProblems);
   if (num_tokens < 0) return fail(LORAX_EINVAL, "num_tokens=%lld is negative", (long long)num_tokens);
   if (num_problems == 0 || num_tokens == 0) return LORAX_OK;
   if (problems == nullptr) return fail(LORAX_EINVAL, "null pointer argument (problems)");
@@ -317,7 +323,7 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
                   (long long)q.y_stride, q.h_out);
     if (q.num_groups > a.grid_rows) a.grid_rows = q.num_groups;
     if (q.h_out > a.wide_max) a.wide_max = q.h_out;
-    a.batch.p[i] = BgmvProblem{q.y, q.x, nullptr, nullptr, q.y_offset, q.y_stride, q.h_out, q.plan, q.num_groups};
+    a.batch.p[i] = BgmvProblem{q.y, q.x, nullptr, nullptr, q.y_offset, q.y_stride, q.h_out, r, q.plan, q.num_groups};
   }
   if (a.grid_rows == 0) return LORAX_OK;
   const hipError_t e = launch_bgmv_lora(a, static_cast<hipStream_t>(stream));

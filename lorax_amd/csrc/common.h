@@ -187,6 +187,14 @@ __device__ __forceinline__ VirtualBlock xcd_virtual_block() {
   return b;
 }
 
+// The same for a one-dimensional grid: consecutive virtual ids run on one XCD.
+__device__ __forceinline__ unsigned xcd_virtual_id() {
+  const unsigned n = gridDim.x;
+  const unsigned per = n / kXcds, rem = n % kXcds;
+  const unsigned xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+  return xcd * per + (xcd < rem ? xcd : rem) + slot;
+}
+
 // Token grouping for BGMV.  Tokens that share an indices[] value share one adapter; the
 // tokens of one adapter are cut, in token order, into chunks of at most G and the
 // first token of each chunk ("leader") processes the whole chunk, so the adapter's

@@ -10,8 +10,8 @@
 namespace lorax {
 
 // One BGMV problem of a batched launch: its own output, input, pointer table and routing.
-// `width` is the problem's wide dimension (h_out of an expand); shrink problems of one
-// launch share h_in and rank, expand problems share the rank.
+// `width` is the problem's wide dimension (h_out of an expand, the shared h_in of a shrink) and
+// `narrow` its LoRA rank; problems of one launch may differ in rank.
 struct BgmvProblem {
   void* y;
   const void* x;
@@ -20,22 +20,36 @@ struct BgmvProblem {
   int64_t y_offset;
   int64_t y_stride;
   int width;
+  int narrow;
   const int64_t* plan;  // optional routing plan: num_groups records of kPlanRecordWords int64
   int num_groups;
 };
 
-constexpr int kMaxBgmvProblems = 4;
+constexpr int kMaxBgmvProblems = 16;
+constexpr int kMaxFusedBgmvProblems = 4;  // the single-launch shrink+expand keeps its batch small
 constexpr int kPlanRecordWords = 8;
 
+// Workgroup numbering of the shrink and expand launches (one-dimensional grid).  Consecutive problems
+// with the same number of token chunks (the projections of one rank group: same routing) form a run.  A
+// run owns the ids [base, run_end); inside it an id is chunk * run_subs + s, and s in [sub_lo[i], sub_hi[i])
+// is row block / column slice s - sub_lo[i] of problem i.  All workgroups of one token chunk are then
+// neighbours - on one XCD, sharing the chunk's input rows through its L2 - and every launched workgroup
+// has a problem, a chunk and a slice of its own, whatever the mix of ranks, widths and routings.
 struct BgmvBatch {
   BgmvProblem p[kMaxBgmvProblems];
+  int run_end[kMaxBgmvProblems];
+  int base[kMaxBgmvProblems];
+  int run_subs[kMaxBgmvProblems];
+  int sub_lo[kMaxBgmvProblems];
+  int sub_hi[kMaxBgmvProblems];
 };
 
 struct BgmvArgs {
   BgmvBatch batch;
   int count;          // problems in the batch (grid z)
   bool expand;        // bgmv_impl.cuh:204: h_in < h_out
-  int narrow;         // LoRA rank
+  int narrow;         // largest LoRA rank of the batch (the fused kernel: the rank)
+  int narrow_sum;     // sum of the problems' ranks
   int wide_max;       // shrink: h_in; expand and fused: widest h_out of the batch
   int h_in;           // fused shrink+expand only: hidden size of x
   int64_t num_tokens;
@@ -81,7 +95,9 @@ struct Tuning {
   int shrink_no_rotate;
   int shrink_lds;  // LORAX_SHRINK_LDS: 1 = always take the LDS-staged shrink where it applies, -1 = never
   int shrink_lds_kb;  // LORAX_SHRINK_LDS_KB: LDS budget of the staged shrink's buffers
+  int bgmv_expand_cols;  // LORAX_BGMV_EXPAND_COLS: columns per lane group of the BGMV expand (4, 8, 16)
   int expand_panels;  // LORAX_EXPAND_PANELS: column panels per wave of the transposed-B expand
+  int bgmv_no_runs;   // LORAX_BGMV_NO_RUNS: number workgroups problem by problem
 };
 const Tuning& tuning();
 

@@ -135,7 +135,8 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
 
 template <typename D, int KS>
 static hipError_t launch_expand_t_ks(const SgmvArgs& a, hipStream_t stream) {
-  int rows_per_tile = a.num_tokens >= 8192 ? 512 : 256;
+  // 256-row tiles: the prologue is one memory round trip, so taller tiles buy nothing and even out worse
+  int rows_per_tile = 256;
   if (tuning().expand_rows > 0) rows_per_tile = (tuning().expand_rows + 15) / 16 * 16;
   const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
   const int num_panels = (a.d_out + kExpTCols - 1) / kExpTCols;

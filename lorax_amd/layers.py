@@ -109,35 +109,48 @@ class LoraLinear(nn.Module):
                         result, v, rs.tmp_expand, rs.lora_b_ptr, rs.segment_starts, rs.segment_ends, self.layer_id
                     )
 
-        step = _native.MAX_BGMV_PROBLEMS
-        for r, jobs in decode_jobs.items():
-            if not tensor_parallel:
-                # small slabs: shrink and expand in one launch, v never leaves the chip
-                single = [j for j in jobs if j[0].plan is not None and _native.bgmv_lora_fits(r, input.size(1), j[2])]
-                jobs = [j for j in jobs if not any(j is s for s in single)]
+        # Decode.  When every job of the call has a small A slab (rank 8 or 16, moderate widths), shrink and
+        # expand run in one launch per rank and v never leaves the chip.  Otherwise all rank groups of all
+        # projections go out together: one shrink launch and one expand launch per 16 problems, whatever the
+        # mix of ranks (the reference issues a pair of launches per projection and rank, layers.py:146-164).
+        jobs = [(r, rs, start, width) for r, rank_jobs in decode_jobs.items() for rs, start, width in rank_jobs]
+        all_fused = bool(jobs) and not tensor_parallel and all(
+            rs.plan is not None and _native.bgmv_lora_fits(r, input.size(1), width) for r, rs, _, width in jobs
+        )
+        if all_fused:
+            step = _native.MAX_FUSED_BGMV_PROBLEMS
+            for r in decode_jobs:
+                single = [j for j in jobs if j[0] == r]
                 for i in range(0, len(single), step):
                     _native.bgmv_lora_multi(
-                        [(result, input, rs.plan, start, width) for rs, start, width in single[i : i + step]],
+                        [(result, input, rs.plan, start, width) for _, rs, start, width in single[i : i + step]],
                         r, self.layer_id,
                     )
-            for i in range(0, len(jobs), step):
-                chunk = jobs[i : i + step]
-                # v needs no zero-fill: the shrink overwrites the rows of routed tokens and the
-                # expand reads no others
-                vs = torch.empty((len(chunk), input.size(0), r), dtype=input.dtype, device=input.device).unbind(0)
-                plans = [rs.plan for rs, _, _ in chunk]
-                if any(p is None for p in plans):
-                    plans = None  # tables not built by BatchLoraWeights.load: the kernels group tokens themselves
-                _native.bgmv_multi(
-                    [(v, input, rs.lora_a_ptr, rs.indices, 0, None) for v, (rs, _, _) in zip(vs, chunk)],
-                    self.layer_id, 1.0, accumulate=False, plans=plans,
-                )
-                if tensor_parallel:
-                    vs = [self.collect_lora_a(v) for v in vs]
-                _native.bgmv_multi(
-                    [(result, v, rs.lora_b_ptr, rs.indices, start, width) for v, (rs, start, width) in zip(vs, chunk)],
-                    self.layer_id, 1.0, accumulate=True, plans=plans,
-                )
+            return result
+        step = _native.MAX_BGMV_PROBLEMS
+        for i in range(0, len(jobs), step):
+            chunk = jobs[i : i + step]
+            # v needs no zero-fill: the shrink overwrites the rows of routed tokens and the expand reads
+            # no others.  One buffer, one [T, r] slice of it per problem.
+            widths = [r for r, _, _, _ in chunk]
+            flat = torch.empty((input.size(0) * sum(widths),), dtype=input.dtype, device=input.device)
+            vs, pos = [], 0
+            for r in widths:
+                vs.append(flat[pos : pos + input.size(0) * r].view(input.size(0), r))
+                pos += input.size(0) * r
+            plans = [rs.plan for _, rs, _, _ in chunk]
+            if any(p is None for p in plans):
+                plans = None  # tables not built by BatchLoraWeights.load: the kernels group tokens themselves
+            _native.bgmv_multi(
+                [(v, input, rs.lora_a_ptr, rs.indices, 0, None) for v, (_, rs, _, _) in zip(vs, chunk)],
+                self.layer_id, 1.0, accumulate=False, plans=plans,
+            )
+            if tensor_parallel:
+                vs = [self.collect_lora_a(v) for v in vs]
+            _native.bgmv_multi(
+                [(result, v, rs.lora_b_ptr, rs.indices, start, width) for v, (_, rs, start, width) in zip(vs, chunk)],
+                self.layer_id, 1.0, accumulate=True, plans=plans,
+            )
         return result
 
     def forward_layer_type(

@@ -230,10 +230,62 @@ def test_bgmv_multi_matches_separate_launches(r):
         routed = idx >= 0
         assert torch.isfinite(v.cpu()[routed].float()).all()
         assert torch.isnan(v.cpu()[~routed].float()).all()  # rows without adapter are not written
-    with pytest.raises(RuntimeError, match="share direction and rank"):
-        _native.bgmv_multi([shrink[0], (torch.zeros((T, r + 8), dtype=dtype, device=DEV),) + shrink[1][1:]], 1)
-    with pytest.raises(RuntimeError, match="between 1 and 4"):
-        _native.bgmv_multi(shrink + shrink, 1)
+    with pytest.raises(RuntimeError, match="share the direction"):
+        _native.bgmv_multi([shrink[0], expand[0]], 1)
+    with pytest.raises(RuntimeError, match="between 1 and 16"):
+        _native.bgmv_multi(shrink * 6, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("use_plan", [False, True])
+def test_bgmv_multi_mixed_ranks(dtype, use_plan):
+    """The rank groups of a multi-rank batch in one shrink launch and one expand launch: every problem has
+    its own rank, routing (a token belongs to exactly one rank group), pointer tables and column window."""
+    from lorax_amd import _native
+    from lorax_amd.adapters import build_bgmv_plan
+
+    T, h_in, n = 150, 2048, 5
+    ranks = [8, 16, 32, 64, 128, 24, 8]
+    sizes = [1024, 512, 1160, 1024, 256, 136, 1024]  # windows of one wide y
+    gen = torch.Generator().manual_seed(77)
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    y0 = randn((T, sum(sizes)), 0.5, gen, dtype, DEV)
+    y, y_ref = y0.clone(), y0.cpu().clone()
+    group_of_token = torch.randint(-1, len(ranks), (T,), generator=gen)  # -1: no adapter at all
+    shrink, expand, plans, keep_alive, vs = [], [], [], [], []
+    off = 0
+    for p, (r, h_out) in enumerate(zip(ranks, sizes)):
+        wa_t = _stacks(n, 2, r, h_in, gen, dtype)
+        wb_t = _stacks(n, 2, h_out, r, gen, dtype)
+        keep_alive.append((wa_t, wb_t))
+        idx = torch.where(group_of_token == p, torch.randint(0, n, (T,), generator=gen), torch.full((T,), -1))
+        v = torch.full((T, r), float("nan"), dtype=dtype, device=DEV)
+        vs.append((v, idx))
+        a_ptr, b_ptr = ptr_table(wa_t, DEV), ptr_table(wb_t, DEV)
+        shrink.append((v, x, a_ptr, idx.to(DEV), 0, None))
+        expand.append((y, v, b_ptr, idx.to(DEV), off, h_out))
+        records = build_bgmv_plan(idx.tolist(), a_ptr.tolist(), b_ptr.tolist())
+        plans.append(torch.tensor(records, dtype=torch.int64, device=DEV).reshape(-1, 8))
+        v_ref = torch.zeros((T, r), dtype=dtype)
+        O.bgmv_ref(v_ref, x.cpu(), [w.cpu() for w in wa_t], idx.tolist(), 1)
+        part = y_ref[:, off:off + h_out].clone()
+        O.bgmv_ref(part, v_ref, [w.cpu() for w in wb_t], idx.tolist(), 1)
+        y_ref[:, off:off + h_out] = part
+        off += h_out
+    _native.bgmv_multi(shrink, 1, 1.0, accumulate=False, plans=plans if use_plan else None)
+    _native.bgmv_multi(expand, 1, 1.0, accumulate=True, plans=plans if use_plan else None)
+    torch.cuda.synchronize()
+    assert_close(y, y_ref, "mixed-rank batch", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
+    for v, idx in vs:
+        routed = idx >= 0
+        assert torch.isfinite(v.cpu()[routed].float()).all()
+        assert torch.isnan(v.cpu()[~routed].float()).all()
+    untouched = torch.ones_like(y_ref, dtype=torch.bool)
+    off = 0
+    for p, h_out in enumerate(sizes):
+        untouched[group_of_token == p, off:off + h_out] = False
+        off += h_out
+    assert torch.equal(y.cpu()[untouched], y0.cpu()[untouched])
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
