@@ -335,12 +335,47 @@ __device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
 #pragma unroll
   for (int g = 0; g < NT; ++g) yrow[g] = Y + static_cast<int64_t>(toks[g]) * y_stride + y_offset;
 
-  // (1) every B^T vector of the workgroup's column range goes out before the shrink: they do
-  // not depend on v, and being cold they are the long pole of the expand.  Clamped, not predicated.
+  // (1) the first trip of the shrink's operands goes out first: loads return in order and these are
+  // needed first, so the dot products run while the expand's operands are still arriving.
+  float acc[R][NT];
+#pragma unroll
+  for (int j = 0; j < R; ++j)
+#pragma unroll
+    for (int g = 0; g < NT; ++g) acc[j][g] = 0.f;
+  const E* xrow[NT];
+#pragma unroll
+  for (int g = 0; g < NT; ++g) xrow[g] = X + static_cast<int64_t>(toks[g]) * h_in;
+  constexpr int kStep = kBgmvThreads * 8;
+  vec8 xv[kSteps][NT];
+  vec8 av[kSteps][R];
+  auto load_trip = [&](int k) {
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+      // a step past the end re-reads the slab's first chunk and is masked to zero
+      const bool live = k + u * kStep < h_in;
+      const int ku = live ? k + u * kStep : 0;
+#pragma unroll
+      for (int g = 0; g < NT; ++g) xv[u][g] = keep_if<D>(live, load8<D>(xrow[g] + ku));
+#pragma unroll
+      for (int j = 0; j < R; ++j) av[u][j] = load8<D>(A + static_cast<int64_t>(j) * h_in + ku);
+    }
+  };
+  auto dot_trip = [&]() {
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u)
+#pragma unroll
+      for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int g = 0; g < NT; ++g) acc[j][g] = dot8<D>(av[u][j], xv[u][g], acc[j][g]);
+  };
+  load_trip(tid * 8);
+
+  // (2) every B^T vector of the workgroup's column range and the old y: they do not depend on v, and
+  // being cold they are the long pole of the expand.  Clamped, not predicated.
   // VEC4 (every y row 8-byte aligned, h_out a multiple of 4): a lane owns U = 4 adjacent columns, so
   // the old y of a block is one 8-byte load per token and the new y one 8-byte store, and all of it
-  // is fetched here, ahead of the shrink.  Otherwise lanes take columns kCols apart and y moves
-  // element by element, one block ahead of the arithmetic.
+  // is fetched here, ahead of the shrink's arithmetic.  Otherwise lanes take columns kCols apart and
+  // y moves element by element, one block ahead of the arithmetic.
   typedef E vec4 __attribute__((ext_vector_type(4)));
   static_assert(!VEC4 || U == 4, "the vector path moves four columns per lane");
   auto column = [&](int blk, int u) {
@@ -371,36 +406,13 @@ __device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
     }
   };
 
-  // (2) shrink: all R rows of the slab against the chunk's tokens
-  float acc[R][NT];
-#pragma unroll
-  for (int j = 0; j < R; ++j)
-#pragma unroll
-    for (int g = 0; g < NT; ++g) acc[j][g] = 0.f;
-  const E* xrow[NT];
-#pragma unroll
-  for (int g = 0; g < NT; ++g) xrow[g] = X + static_cast<int64_t>(toks[g]) * h_in;
-  constexpr int kStep = kBgmvThreads * 8;
-  for (int k = tid * 8; k < h_in; k += kSteps * kStep) {
-    vec8 xv[kSteps][NT];
-    vec8 av[kSteps][R];
-#pragma unroll
-    for (int u = 0; u < kSteps; ++u) {
-      // a step past the end re-reads the thread's first chunk and is masked to zero below
-      const bool live = k + u * kStep < h_in;
-      const int ku = live ? k + u * kStep : tid * 8;
-#pragma unroll
-      for (int g = 0; g < NT; ++g) xv[u][g] = keep_if<D>(live, load8<D>(xrow[g] + ku));
-#pragma unroll
-      for (int j = 0; j < R; ++j) av[u][j] = load8<D>(A + static_cast<int64_t>(j) * h_in + ku);
-    }
+  // shrink: all R rows of the slab against the chunk's tokens
+  __builtin_amdgcn_sched_barrier(0);
+  dot_trip();
+  for (int k = tid * 8 + kSteps * kStep; k < h_in; k += kSteps * kStep) {
+    load_trip(k);
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int u = 0; u < kSteps; ++u)
-#pragma unroll
-      for (int j = 0; j < R; ++j)
-#pragma unroll
-        for (int g = 0; g < NT; ++g) acc[j][g] = dot8<D>(av[u][j], xv[u][g], acc[j][g]);
+    dot_trip();
   }
 
   // (3) workgroup-wide sums -> v in LDS, rounded to the storage type

@@ -36,7 +36,8 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     typename D::E* __restrict__ Y, const typename D::E* __restrict__ V,
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int r, int h_out,
-    int64_t y_offset, int64_t y_stride, int64_t layer_idx, int rows_per_tile, int panels_per_wave) {
+    int64_t y_offset, int64_t y_stride, int64_t layer_idx, int rows_per_tile, int panels_per_wave,
+    int tile_slots) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   const int lane = threadIdx.x & (kWave - 1);
@@ -44,7 +45,11 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
   const int c = lane & 15;
   const int g = lane >> 4;
   const int num_panels = (h_out + kExpTCols - 1) / kExpTCols;
-  const int panel0 = blockIdx.x * kExpTWaves * panels_per_wave;
+  // Workgroup numbering: row tiles fastest, then panel groups, and consecutive numbers on one XCD.  The
+  // row tiles of a long segment read the same panels of B^T; as neighbours on one XCD they find them in
+  // its L2 instead of fetching them once per tile.
+  const int vid = static_cast<int>(xcd_virtual_id());
+  const int panel0 = (vid / tile_slots) * kExpTWaves * panels_per_wave;
 
   bool k_ok[KS];
   int k_off[KS];
@@ -54,7 +59,7 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     k_off[s] = k_ok[s] ? s * 32 + g * 8 : 0;
   }
 
-  for (int tile = blockIdx.y;; tile += gridDim.y) {
+  for (int tile = vid % tile_slots;; tile += tile_slots) {
     RowTile rt;
     if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const E* BT = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * h_out * static_cast<int64_t>(r);
@@ -145,12 +150,13 @@ static hipError_t launch_expand_t_ks(const SgmvArgs& a, hipStream_t stream) {
   int ppw = 4;
   while (ppw > 1 && tiles * ((num_panels + kExpTWaves * ppw - 1) / (kExpTWaves * ppw)) < 4096) ppw /= 2;
   if (tuning().expand_panels > 0) ppw = tuning().expand_panels;
-  dim3 grid((num_panels + kExpTWaves * ppw - 1) / (kExpTWaves * ppw),
-            static_cast<unsigned>(tiles < 65535 ? tiles : 65535));
+  const int64_t panel_groups = (num_panels + kExpTWaves * ppw - 1) / (kExpTWaves * ppw);
+  const int tile_slots = static_cast<int>(tiles < 65535 ? tiles : 65535);
+  dim3 grid(static_cast<unsigned>(panel_groups * tile_slots));
   hipLaunchKernelGGL((sgmv_expand_t_kernel<D, KS>), grid, dim3(kExpTThreads), 0, stream,
                      static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start,
                      a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.y_offset,
-                     a.y_stride, a.layer_idx, rows_per_tile, ppw);
+                     a.y_stride, a.layer_idx, rows_per_tile, ppw, tile_slots);
   return hipGetLastError();
 }
 
