@@ -116,6 +116,10 @@ struct BatchSlot {
 };
 __device__ __forceinline__ BatchSlot batch_slot(const BgmvBatch& batch, int count) {
   const int v = static_cast<int>(xcd_virtual_id());
+  if (count == 1) {  // the drop-in single-problem call: no table walk in front of the first useful load
+    const int subs = batch.run_subs[0];
+    return BatchSlot{0, v / subs, v % subs};
+  }
   int p = 0;
   while (p + 1 < count && v >= batch.run_end[p]) ++p;  // first problem of the run that holds v
   const int rem = v - batch.base[p];
@@ -624,6 +628,7 @@ static hipError_t launch_expand(const BgmvArgs& a, hipStream_t stream) {
   for (int i = 0; i < a.count; ++i)
     bytes += a.work_rows * a.batch.p[i].width * static_cast<int64_t>(a.batch.p[i].narrow) * 2;
   int u = bytes >= (32ll << 20) ? 4 : 2;
+  if (a.batch.p[0].plan == nullptr) u = 4;  // every workgroup scans indices[] for its chunk: fewer of them
   if (tuning().bgmv_expand_cols > 0) u = tuning().bgmv_expand_cols;
   if (u >= 8) return launch_expand_u<D, 8>(a, stream);
   if (u <= 2) return launch_expand_u<D, 2>(a, stream);
