@@ -130,18 +130,23 @@ class Plan:
         v = torch.zeros((x.size(0), r), dtype=x.dtype, device=x.device)
         lens = (rd.segment_ends - rd.segment_starts).clamp(min=0)
         rows = int(lens.sum().item())
-        uniq = len(set(rd.lora_a_ptr[lens > 0].tolist()))
+        uniq = len(set(rd.lora_a_t_ptr[lens > 0].tolist()))
         starts, ends, tmp_s, tmp_e = rd.segment_starts, rd.segment_ends, rd.tmp_shrink, rd.tmp_expand
-        a_ptr, b_ptr = rd.lora_a_ptr, rd.lora_b_ptr
-        a_is_rh = not sgmv.use_cutlass_shrink(r)
+        fused = self.pattern == "fused"
+        resident_a = fused and sgmv.resident_shrink_applies(r, h_in)
+        # the layers' pattern reads the resident stacks; the reference pattern its prefill layouts
+        a_ptr = rd.lora_a_t_ptr if resident_a else rd.lora_a_ptr
+        b_ptr = None if fused else rd.lora_b_ptr
+        bt_ptr = rd.lora_b_t_ptr if fused else None
+        a_is_rh = resident_a or not sgmv.use_cutlass_shrink(r)
+        if a_is_rh:
+            tmp_s = sgmv.get_tmp_tensor(x.device)
 
         def shrink(layer):
             if a_is_rh:
                 sgmv._kernels.sgmv_shrink(v, x, a_ptr, starts, ends, tmp_s, layer)
             else:
                 sgmv._kernels.sgmv_cutlass(v, x, a_ptr, starts, ends, tmp_s, layer)
-
-        bt_ptr = rd.lora_b_t_ptr if self.pattern == "fused" else None
 
         def expand(layer):
             if bt_ptr is not None:

@@ -150,8 +150,8 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
  *   empty or negative segments are skipped without reading w_ptrs[i]
  *   (sgmv_cutlass.cuh:39-44).  Rows at or beyond num_tokens are never accessed.
  *
- * r must be a multiple of 16 in [16, 128] for LORAX_A_RH and 8 or a multiple of 16
- * up to 128 for LORAX_A_HR; h_in a multiple of 8.  `tmp`/`tmp_bytes` is the caller's
+ * r must be a multiple of 8 in [8, 128]; h_in a multiple of 8; LORAX_A_RH with a rank that is not a
+ * multiple of 16 additionally needs h_in to be a multiple of 128.  `tmp`/`tmp_bytes` is the caller's
  * scratch and is only validated for presence; the split-K partial sums live in the
  * library's own per-device workspace (see lorax_init).
  */

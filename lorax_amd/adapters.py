@@ -12,6 +12,7 @@ Attribute and method names are the reference's, so its LoRA layer code and its t
 
 from abc import ABC, abstractmethod
 from collections import defaultdict
+from collections.abc import Mapping
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Set, Tuple, Type
 
@@ -92,15 +93,16 @@ def get_scaling_factor(lora_alpha: int, r: int, uses_rslora: bool = False) -> fl
 class LoraWeights(AdapterWeights):
     """One adapter's A and B for one layer type, stacked over layers (adapters/lora.py:87-140).
 
-    Constructed from per-layer ``A: [h_in, r]`` and ``B: [r, h_out]``.  Two layouts:
-      prefill (SGMV): weights_a = [L, r, h_in] for 16 <= r <= 128, else [L, h_in, r];
-                      weights_b = [L, r, h_out]
-      decode  (BGMV): weights_a_t = [L, r, h_in]; weights_b_t = [L, h_out, r]
-    The reference keeps one layout at a time and re-transposes the whole stack whenever a batch
-    of the other kind arrives (adapters/lora.py:111-140), which also moves the stack to a new
-    address.  Here the second layout is materialised on first use and then both stay resident,
-    so every pointer handed to the kernels stays valid for the adapter's lifetime; with 288 GB
-    of HBM the extra copy of B (and of A below rank 16) is the cheaper side of that trade.
+    Constructed from per-layer ``A: [h_in, r]`` and ``B: [r, h_out]``.  ONE resident layout serves
+    both kernels families here:
+      weights_a_t = [L, r, h_in]   read by BGMV shrink and by SGMV shrink (any rank multiple of 8)
+      weights_b_t = [L, h_out, r]  read by BGMV expand and by SGMV expand
+    The reference keeps one of two layouts at a time - prefill: weights_a = [L, r, h_in] for
+    16 <= r <= 128 else [L, h_in, r], weights_b = [L, r, h_out]; decode: the two above - and
+    re-transposes the whole stack whenever a batch of the other kind arrives (adapters/lora.py:111-140),
+    which also moves the stack to a new address.  weights_a / weights_b are still available for
+    callers of the reference-layout entry points; they are materialised on first use and then stay
+    resident too, so every pointer handed to the kernels stays valid for the adapter's lifetime.
     """
 
     def __init__(self, weights_a: List[torch.Tensor], weights_b: List[torch.Tensor], adapter_config: LoraConfig):
@@ -108,32 +110,34 @@ class LoraWeights(AdapterWeights):
         self.lora_a_r = weights_a[0].size(1) if has_layers else 1
         self.lora_b_r = weights_b[0].size(0) if has_layers else 1
         self._use_cutlass_shrink = use_cutlass_shrink(self.lora_a_r)
-        self._weights_a = torch.stack([orient_for_rank(w, w.size(1)).contiguous() for w in weights_a])
-        self._weights_b = torch.stack(list(weights_b))
-        self._weights_a_t: Optional[torch.Tensor] = None
-        self._weights_b_t: Optional[torch.Tensor] = None
+        self._weights_a_t = torch.stack([w.transpose(0, 1).contiguous() for w in weights_a])  # [L, r, h_in]
+        self._weights_b_t = torch.stack([w.transpose(0, 1).contiguous() for w in weights_b])  # [L, h_out, r]
+        self._weights_a: Optional[torch.Tensor] = None
+        self._weights_b: Optional[torch.Tensor] = None
         self.adapter_config = adapter_config
 
     @property
     def weights_a(self) -> torch.Tensor:
+        """The reference's prefill layout of A (orient_for_rank, punica.py:83-86)."""
+        if self._weights_a is None:
+            # only below rank 16 do the two layouts disagree about A
+            a = self._weights_a_t
+            self._weights_a = a.transpose(1, 2).contiguous() if self._use_cutlass_shrink else a
         return self._weights_a
 
     @property
     def weights_b(self) -> torch.Tensor:
+        """The reference's prefill layout of B, [L, r, h_out]."""
+        if self._weights_b is None:
+            self._weights_b = self._weights_b_t.transpose(1, 2).contiguous()
         return self._weights_b
 
     @property
     def weights_a_t(self) -> torch.Tensor:
-        if self._weights_a_t is None:
-            # only below rank 16 do the two layouts disagree about A
-            a = self._weights_a
-            self._weights_a_t = a.transpose(1, 2).contiguous() if self._use_cutlass_shrink else a
         return self._weights_a_t
 
     @property
     def weights_b_t(self) -> torch.Tensor:
-        if self._weights_b_t is None:
-            self._weights_b_t = self._weights_b.transpose(1, 2).contiguous()
         return self._weights_b_t
 
     @classmethod
@@ -158,28 +162,49 @@ class LoraWeights(AdapterWeights):
         return cls(a_list, b_list, config)
 
 
-@dataclass
 class RankSegments:
-    """Kernel arguments of one rank group (adapters/lora.py:213-227)."""
+    """Kernel arguments of one rank group (adapters/lora.py:213-227).
 
-    rank: int
-    lora_a_ptr: torch.Tensor
-    lora_b_ptr: torch.Tensor
-    # prefill (SGMV)
-    tmp_shrink: Optional[torch.Tensor]
-    tmp_expand: Optional[torch.Tensor]
-    segment_starts: Optional[torch.Tensor]
-    segment_ends: Optional[torch.Tensor]
-    # decode (BGMV)
-    indices: Optional[torch.Tensor]
-    # decode: routing plan for the batched BGMV launches, int64 [num_chunks, 8] on the device; one record
-    # per chunk of up to BGMV_PLAN_GROUP tokens of one adapter: [count, tok0..tok3, address of the A stack,
-    # address of the B^T stack, 0]. Derived from `indices` and the pointer tables; no counterpart in the
-    # reference, whose kernels take one token per thread block.
-    plan: Optional[torch.Tensor] = None
-    # prefill: addresses of the transposed B stacks ([L, h_out, r], weights_b_t - the stacks decode uses), one per
-    # segment like lora_b_ptr; the expand kernel for this layout reads each column panel as one contiguous run.
-    lora_b_t_ptr: Optional[torch.Tensor] = None
+    lora_a_ptr / lora_b_ptr are the reference's tables: in decode the addresses of the [L, r, h_in] and
+    [L, h_out, r] stacks, in prefill those of the reference's prefill layouts.  The prefill kernels here read
+    the decode stacks too (lora_a_t_ptr / lora_b_t_ptr), so the reference-layout tables of a prefill batch -
+    and the weight copies behind them - are only built when somebody asks for them."""
+
+    def __init__(self, rank: int, lora_a_ptr, lora_b_ptr, tmp_shrink: Optional[torch.Tensor],
+                 tmp_expand: Optional[torch.Tensor], segment_starts: Optional[torch.Tensor],
+                 segment_ends: Optional[torch.Tensor], indices: Optional[torch.Tensor],
+                 plan: Optional[torch.Tensor] = None, lora_a_t_ptr: Optional[torch.Tensor] = None,
+                 lora_b_t_ptr: Optional[torch.Tensor] = None):
+        self.rank = rank
+        self._lora_a_ptr = lora_a_ptr  # a tensor, or a function that builds it
+        self._lora_b_ptr = lora_b_ptr
+        # prefill (SGMV)
+        self.tmp_shrink = tmp_shrink
+        self.tmp_expand = tmp_expand
+        self.segment_starts = segment_starts
+        self.segment_ends = segment_ends
+        # decode (BGMV)
+        self.indices = indices
+        # decode: routing plan for the batched BGMV launches, int64 [num_chunks, 8] on the device; one record
+        # per chunk of up to BGMV_PLAN_GROUP tokens of one adapter: [count, tok0..tok3, address of the A stack,
+        # address of the B^T stack, 0]. Derived from `indices` and the pointer tables; no counterpart in the
+        # reference, whose kernels take one token per thread block.
+        self.plan = plan
+        # prefill: addresses of the resident stacks, one per segment like lora_a_ptr / lora_b_ptr
+        self.lora_a_t_ptr = lora_a_t_ptr
+        self.lora_b_t_ptr = lora_b_t_ptr
+
+    @property
+    def lora_a_ptr(self) -> Optional[torch.Tensor]:
+        if callable(self._lora_a_ptr):
+            self._lora_a_ptr = self._lora_a_ptr()
+        return self._lora_a_ptr
+
+    @property
+    def lora_b_ptr(self) -> Optional[torch.Tensor]:
+        if callable(self._lora_b_ptr):
+            self._lora_b_ptr = self._lora_b_ptr()
+        return self._lora_b_ptr
 
 
 BGMV_PLAN_GROUP = 4
@@ -203,6 +228,23 @@ def build_bgmv_plan(token_slots: List[int], a_addrs: List[int], b_addrs: List[in
     return records
 
 
+class _LayoutView(Mapping):
+    """adapter index -> one layout of its stack (an attribute of LoraWeights), fetched on access."""
+
+    def __init__(self, loras: Dict[int, "LoraWeights"], layout: str):
+        self._loras = loras
+        self._layout = layout
+
+    def __getitem__(self, idx: int) -> torch.Tensor:
+        return getattr(self._loras[idx], self._layout)
+
+    def __iter__(self):
+        return iter(self._loras)
+
+    def __len__(self) -> int:
+        return len(self._loras)
+
+
 def _unwrap(weights):
     return weights.lora_weights if hasattr(weights, "lora_weights") else weights
 
@@ -211,8 +253,8 @@ def _unwrap(weights):
 class BatchLoraWeights(BatchAdapterWeights):
     """adapters/lora.py:230-396."""
 
-    lora_a: Dict[int, torch.Tensor]
-    lora_b: Dict[int, torch.Tensor]
+    lora_a: Mapping  # adapter index -> A stack in the reference's prefill layout (built on access)
+    lora_b: Mapping  # adapter index -> B stack [L, r, h_out] (built on access)
     adapter_index_configs: Dict[int, LoraConfig]
     rank_data: Dict[int, RankSegments]
     use_sgmv: bool
@@ -251,28 +293,26 @@ class BatchLoraWeights(BatchAdapterWeights):
         covered = [s for s, idx in enumerate(seg_adapters) if idx in loras]
         if not covered:
             return None
-        device = next(iter(loras.values())).weights_a.device
+        device = next(iter(loras.values())).weights_a_t.device
 
-        lora_a = {seg_adapters[s]: loras[seg_adapters[s]].weights_a for s in covered}
-        lora_b = {seg_adapters[s]: loras[seg_adapters[s]].weights_b for s in covered}
+        # adapter -> stack in the reference's prefill layout, read (and materialised) on access only
+        lora_a = _LayoutView({seg_adapters[s]: loras[seg_adapters[s]] for s in covered}, "weights_a")
+        lora_b = _LayoutView({seg_adapters[s]: loras[seg_adapters[s]] for s in covered}, "weights_b")
         max_rank = max(loras[seg_adapters[s]].lora_a_r for s in covered)
         use_sgmv = bool(prefill or max_rank > BGMV_MAX_RANK)
 
         # One pointer per segment; segments without weights hold a placeholder address that no
         # rank group refers to.
         null = EMPTY_TENSOR.data_ptr()
-        if use_sgmv:
-            a_addr = [loras[i].weights_a.data_ptr() if i in loras else null for i in seg_adapters]
-            b_addr = [loras[i].weights_b.data_ptr() if i in loras else null for i in seg_adapters]
-        else:
-            a_addr = [loras[i].weights_a_t.data_ptr() if i in loras else null for i in seg_adapters]
-            b_addr = [loras[i].weights_b_t.data_ptr() if i in loras else null for i in seg_adapters]
-        lora_a_ptr = torch.tensor(a_addr, dtype=torch.int64, device=device)
-        lora_b_ptr = torch.tensor(b_addr, dtype=torch.int64, device=device)
-        lora_b_t_ptr = None
-        if use_sgmv:
-            bt_addr = [loras[i].weights_b_t.data_ptr() if i in loras else null for i in seg_adapters]
-            lora_b_t_ptr = torch.tensor(bt_addr, dtype=torch.int64, device=device)
+
+        def table(layout: str) -> torch.Tensor:
+            addr = [getattr(loras[i], layout).data_ptr() if i in loras else null for i in seg_adapters]
+            return torch.tensor(addr, dtype=torch.int64, device=device)
+
+        a_addr = [loras[i].weights_a_t.data_ptr() if i in loras else null for i in seg_adapters]
+        b_addr = [loras[i].weights_b_t.data_ptr() if i in loras else null for i in seg_adapters]
+        lora_a_t_ptr = torch.tensor(a_addr, dtype=torch.int64, device=device)
+        lora_b_t_ptr = torch.tensor(b_addr, dtype=torch.int64, device=device)
 
         configs = {seg_adapters[s]: loras[seg_adapters[s]].adapter_config for s in covered}
 
@@ -315,17 +355,24 @@ class BatchLoraWeights(BatchAdapterWeights):
                 token_slots = torch.tensor(slots, dtype=torch.int64, device=device)
                 records = build_bgmv_plan(slots, [a_addr[s] for s in segs], [b_addr[s] for s in segs])
                 plan = torch.tensor(records, dtype=torch.int64, device=device).reshape(-1, BGMV_PLAN_WORDS)
+            if use_sgmv:
+                # the reference's prefill tables, built (with the weight copies behind them) on first access
+                ref_a = (lambda segs=segs: table("weights_a")[segs])
+                ref_b = (lambda segs=segs: table("weights_b")[segs])
+            else:
+                ref_a, ref_b = lora_a_t_ptr[segs], lora_b_t_ptr[segs]
             rank_data[rank] = RankSegments(
                 rank=rank,
-                lora_a_ptr=lora_a_ptr[segs],
-                lora_b_ptr=lora_b_ptr[segs],
+                lora_a_ptr=ref_a,
+                lora_b_ptr=ref_b,
                 tmp_shrink=tmp_shrink,
                 tmp_expand=tmp_expand,
                 segment_starts=starts,
                 segment_ends=ends,
                 indices=token_slots,
                 plan=plan,
-                lora_b_t_ptr=lora_b_t_ptr[segs] if lora_b_t_ptr is not None else None,
+                lora_a_t_ptr=lora_a_t_ptr[segs] if use_sgmv else None,
+                lora_b_t_ptr=lora_b_t_ptr[segs] if use_sgmv else None,
             )
 
         return cls(

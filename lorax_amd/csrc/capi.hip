@@ -219,8 +219,10 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
   if (s_start == nullptr || s_end == nullptr || (tmp == nullptr && tmp_bytes > 0))
     return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p tmp=%p)", s_start, s_end, tmp);
   if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
-  const bool r_ok = a_layout == LORAX_A_RH ? (r >= 16 && r <= kMaxRank && r % 16 == 0)
-                                           : (r >= 8 && r <= kMaxRank && r % 8 == 0);
+  // [L, r, h_in]: multiples of 16 as in the reference (sgmv_config.h:10-15), and any multiple of 8 where the
+  // LDS-staged kernel applies (h_in a multiple of 128)
+  const bool r_ok = r >= 8 && r <= kMaxRank && r % 8 == 0 &&
+                    (a_layout == LORAX_A_HR || r % 16 == 0 || h_in % 128 == 0);
   if (!r_ok || h_in <= 0 || h_in % 8 != 0 || num_tokens > INT32_MAX / 2)
     return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in,
                 r, a_layout);

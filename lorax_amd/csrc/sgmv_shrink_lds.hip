@@ -58,10 +58,12 @@ template <typename D, int NB, int MBLK, bool KSPLIT>
 __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     typename D::E* __restrict__ V, const typename D::E* __restrict__ X,
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
-    const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in,
+    const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int r,
     int64_t layer_idx, int stages) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
+  // NB = ceil(r / 16) rank blocks; the rank itself only needs to be a multiple of 8: rows of the A tile past
+  // the rank re-read the last row and their columns of the result are not stored.
   constexpr int R = NB * 16;
   constexpr int ROWS = MBLK * 16;
   constexpr int kXBytes = ROWS * kLdsRowBytes;
@@ -95,7 +97,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
   for (int tile = vb.x;; tile += gridDim.x) {
     RowTile rt;
     if (!find_row_tile(s_start, s_end, num_segments, num_tokens, ROWS, tile, rt)) break;
-    const E* A = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * R * static_cast<int64_t>(h_in);
+    const E* A = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * r * static_cast<int64_t>(h_in);
 
     // Source addresses of this thread's chunks.  Load j of a thread covers chunk id j * 256 + tid of
     // the tile: row = id / 16, position = id % 16, and it fetches the row's chunk position ^ (row & 15).
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     for (int j = 0; j < kALoads; ++j) {
       const int id = j * kLdsThreads + tid;
       const int row = id >> 4;
-      asrc[j] = A + static_cast<int64_t>(row) * h_in + (((id & 15) ^ (row & 15)) << 3);
+      asrc[j] = A + static_cast<int64_t>(min(row, r - 1)) * h_in + (((id & 15) ^ (row & 15)) << 3);
     }
     auto issue = [&](int st, int slot) {
       char* buf = lds + slot * kStageBytes;
@@ -188,7 +190,8 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
           sum[0] += part[0]; sum[1] += part[1]; sum[2] += part[2]; sum[3] += part[3];
         }
         const int row = rt.row0 + (blk / NB) * 16 + (l & 15);
-        if (row < rt.row_end) accumulate4<D>(V + static_cast<int64_t>(row) * R + (blk % NB) * 16 + 4 * (l >> 4), sum);
+        const int col = (blk % NB) * 16 + 4 * (l >> 4);
+        if (row < rt.row_end && col < r) accumulate4<D>(V + static_cast<int64_t>(row) * r + col, sum);
       }
     } else {
       // every wave owns its output blocks: no cross-wave reduction
@@ -197,8 +200,10 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
         const int row = rt.row0 + (wm * MPW + mb) * 16 + c;
         if (row < rt.row_end) {
 #pragma unroll
-          for (int nb = 0; nb < NPW; ++nb)
-            accumulate4<D>(V + static_cast<int64_t>(row) * R + (wn * NPW + nb) * 16 + 4 * g, acc[mb][nb]);
+          for (int nb = 0; nb < NPW; ++nb) {
+            const int col = (wn * NPW + nb) * 16 + 4 * g;
+            if (col < r) accumulate4<D>(V + static_cast<int64_t>(row) * r + col, acc[mb][nb]);
+          }
         }
       }
     }
@@ -237,7 +242,7 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   dim3 grid(static_cast<unsigned>(tiles < (1 << 20) ? tiles : (1 << 20)));
   hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, static_cast<typename D::E*>(a.y),
                      static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end, a.num_segments,
-                     static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages);
+                     static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, stages);
   return hipGetLastError();
 }
 
@@ -269,7 +274,7 @@ static hipError_t launch_lds_nb(const SgmvArgs& a, hipStream_t stream) {
 
 template <typename D>
 static hipError_t launch_lds_dtype(const SgmvArgs& a, hipStream_t stream) {
-  switch (a.d_out / 16) {
+  switch ((a.d_out + 15) / 16) {
     case 1:
       return launch_lds_nb<D, 1>(a, stream);
     case 2:
@@ -292,7 +297,7 @@ static hipError_t launch_lds_dtype(const SgmvArgs& a, hipStream_t stream) {
 }
 
 bool sgmv_shrink_lds_applies(const SgmvArgs& a) {
-  return a.a_layout == LORAX_A_RH && a.d_in % kLdsKc == 0 && a.d_out % 16 == 0 && a.d_out >= 16 && a.d_out <= 128;
+  return a.a_layout == LORAX_A_RH && a.d_in % kLdsKc == 0 && a.d_out % 8 == 0 && a.d_out >= 8 && a.d_out <= 128;
 }
 
 hipError_t launch_sgmv_shrink_lds(const SgmvArgs& a, hipStream_t stream) {

@@ -28,10 +28,13 @@ from torch import nn
 from lorax_amd import _native
 from lorax_amd.adapters import LORA, AdapterBatchData, BatchLoraWeights
 from lorax_amd.sgmv import (
+    get_tmp_tensor,
     has_sgmv,
     lora_a_sgmv_cutlass,
+    lora_a_sgmv_resident,
     lora_b_sgmv_cutlass,
     lora_b_sgmv_cutlass_slice,
+    resident_shrink_applies,
 )
 
 
@@ -83,18 +86,26 @@ class LoraLinear(nn.Module):
                 continue
             sliced = end - start != result.shape[1]
             for r, rs in data.rank_data.items():
-                if rs.lora_a_ptr is None or rs.lora_b_ptr is None:
-                    continue
                 if not data.use_sgmv:
+                    if rs.lora_a_ptr is None or rs.lora_b_ptr is None:
+                        continue
                     decode_jobs[r].append((rs, start, end - start))
                     continue
-                v = lora_a_sgmv_cutlass(
-                    input, rs.tmp_shrink, rs.lora_a_ptr, rs.segment_starts, rs.segment_ends, self.layer_id, r
-                )
+                # Prefill reads the resident stacks ([L, r, h_in] and [L, h_out, r], the ones decode uses);
+                # the reference's prefill layouts are only touched for shapes the resident-layout shrink
+                # does not take.
+                if rs.lora_a_t_ptr is not None and resident_shrink_applies(r, input.size(1)):
+                    v = lora_a_sgmv_resident(
+                        input, get_tmp_tensor(input.device), rs.lora_a_t_ptr, rs.segment_starts, rs.segment_ends,
+                        self.layer_id, r,
+                    )
+                else:
+                    v = lora_a_sgmv_cutlass(
+                        input, rs.tmp_shrink, rs.lora_a_ptr, rs.segment_starts, rs.segment_ends, self.layer_id, r
+                    )
                 if tensor_parallel:
                     v = self.collect_lora_a(v)
                 if rs.lora_b_t_ptr is not None:
-                    # transposed B stacks (resident for decode anyway): the faster expand
                     lora_b_sgmv_cutlass_slice(
                         result, v, rs.tmp_expand, rs.lora_b_t_ptr, rs.segment_starts, rs.segment_ends,
                         self.layer_id, start, end - start, transposed=True,

@@ -133,6 +133,28 @@ def lora_a_sgmv_cutlass(
     return v
 
 
+def lora_a_sgmv_resident(
+    x: torch.Tensor,
+    tmp: torch.Tensor,
+    wa_t_ptr: torch.Tensor,
+    s_start: torch.IntTensor,
+    s_end: torch.IntTensor,
+    layer_idx: int,
+    lora_rank: int,
+) -> torch.Tensor:
+    """As lora_a_sgmv_cutlass, reading the [L, r, h_in] stacks of the decode path (weights_a_t) whatever
+    the rank.  `tmp` is the 8 MiB buffer of get_tmp_tensor."""
+    v = torch.zeros((x.size(0), lora_rank), dtype=x.dtype, device=x.device)
+    _native_module().sgmv_shrink(v, x, wa_t_ptr, s_start, s_end, tmp, layer_idx)
+    return v
+
+
+def resident_shrink_applies(lora_rank: int, h_in: int) -> bool:
+    """Ranks the [L, r, h_in] shrink entry accepts: multiples of 16 always, other multiples of 8 when h_in is
+    a multiple of 128."""
+    return 8 <= lora_rank <= MAX_RANK_CUSTOM and lora_rank % 8 == 0 and (lora_rank % 16 == 0 or h_in % 128 == 0)
+
+
 def lora_b_sgmv_cutlass(
     y: torch.Tensor,
     v: torch.Tensor,

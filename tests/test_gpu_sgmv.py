@@ -207,6 +207,45 @@ def test_sgmv_expand_transposed_b(dtype, r, h_out, lens, window):
     assert torch.equal(y_t.cpu()[outside], y0.cpu()[outside])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("r", [8, 24, 40, 72, 120])
+@pytest.mark.parametrize("h_in,lens", [(1024, [1, 0, 3, 17, 1, 64, 5, 0, 130]), (256, [700, 650, 3, 900])])
+def test_sgmv_shrink_resident_layout_any_rank(dtype, r, h_in, lens):
+    """lorax_sgmv_shrink with LORAX_A_RH stacks ([L, r, h_in]) takes every rank that is a multiple of 8 when
+    h_in is a multiple of 128 - the layout decode keeps resident, so prefill needs no second copy of A."""
+    print(f"case dtype={dtype} r={r} h_in={h_in} lens={lens}", flush=True)
+    from lorax_amd import _native
+
+    gen = torch.Generator().manual_seed(r + h_in)
+    starts, ends, pos = [], [], 0
+    for n in lens:
+        starts.append(pos)
+        ends.append(pos + n)
+        pos += n + 1  # one uncovered row after every segment
+    T = pos
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    wa_t = [randn((2, r, h_in), 0.05, gen, dtype, DEV) if n > 0 else None for n in lens]
+    v = torch.zeros((T, r), dtype=dtype, device=DEV)
+    _native.sgmv_shrink(v, x, ptr_table(wa_t, DEV), torch.tensor(starts, dtype=torch.int32, device=DEV),
+                        torch.tensor(ends, dtype=torch.int32, device=DEV), sgmv.get_tmp_tensor(torch.device(DEV)), 1)
+    torch.cuda.synchronize()
+    v_ref = torch.zeros((T, r), dtype=dtype)
+    for i, (s, e) in enumerate(zip(starts, ends)):
+        if e > s:
+            v_ref[s:e] = x.cpu()[s:e] @ wa_t[i][1].cpu().t()
+    assert_close(v, v_ref, "shrink output v")
+    covered = torch.zeros(T, dtype=torch.bool)
+    for s, e in zip(starts, ends):
+        covered[s:e] = True
+    assert torch.count_nonzero(v.cpu()[~covered]) == 0
+    if r % 16 != 0:
+        with pytest.raises(RuntimeError, match="No suitable kernel"):
+            _native.sgmv_shrink(torch.zeros((T, r), dtype=dtype, device=DEV), x[:, :h_in - 64].contiguous(),
+                                ptr_table(wa_t, DEV), torch.tensor(starts, dtype=torch.int32, device=DEV),
+                                torch.tensor(ends, dtype=torch.int32, device=DEV),
+                                sgmv.get_tmp_tensor(torch.device(DEV)), 1)
+
+
 @pytest.mark.parametrize("r", [48, 80, 96, 112])
 def test_sgmv_other_multiples_of_16(r):
     """pad_to_min_rank can produce these ranks (punica.py:57-65); the reference's shrink has no

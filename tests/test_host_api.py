@@ -277,3 +277,31 @@ def test_decode_rank_groups_carry_a_plan(case):
         for rec in rd.plan.tolist():
             s = idx[rec[1]]
             assert rec[5] == rd.lora_a_ptr[s].item() and rec[6] == rd.lora_b_ptr[s].item()
+
+
+def test_prefill_tables_touch_only_resident_layouts():
+    """Building the tables of a prefill batch must not materialise the reference's prefill layouts: the kernels
+    read the resident [L, r, h_in] / [L, h_out, r] stacks; the reference-layout tables appear on first access."""
+    from lorax_amd.adapters import BatchLoraWeights, LayerAdapterWeights, LoraConfig, LoraWeights
+    from lorax_amd.synthetic import make_meta
+
+    h, L = 32, 2
+    layer = LayerAdapterWeights()
+    for idx, r in ((0, 8), (1, 16)):
+        a = [torch.randn(h, r) for _ in range(L)]
+        b = [torch.randn(r, h) for _ in range(L)]
+        layer.add_adapter(idx, LoraWeights(a, b, LoraConfig(r=r)))
+    meta = make_meta([0, 0, 1, 1, 1, 0], torch.device("cpu"))
+    data = BatchLoraWeights.load(layer.adapter_weights, meta, "q_proj", prefill=True, prefill_head_indices=None)
+    lws = [layer.adapter_weights[i] for i in (0, 1)]
+    assert all(lw._weights_a is None and lw._weights_b is None for lw in lws)
+    for r, rd in data.rank_data.items():
+        owner = lws[0] if r == 8 else lws[1]
+        assert set(rd.lora_a_t_ptr.tolist()) == {owner.weights_a_t.data_ptr()}
+        assert set(rd.lora_b_t_ptr.tolist()) == {owner.weights_b_t.data_ptr()}
+    assert all(lw._weights_a is None and lw._weights_b is None for lw in lws)
+    rd8 = data.rank_data[8]
+    assert set(rd8.lora_a_ptr.tolist()) == {lws[0].weights_a.data_ptr()}  # now the [L, h_in, 8] copy exists
+    assert lws[0].weights_a.shape == (L, h, 8) and lws[0].weights_a_t.shape == (L, 8, h)
+    assert data.lora_b[1].shape == (L, 16, h) and lws[1]._weights_b is not None
+    assert torch.equal(lws[0].weights_a.transpose(1, 2), lws[0].weights_a_t)
