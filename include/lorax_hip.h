@@ -149,6 +149,8 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
  *     v[s_start[i]:s_end[i], :] += dtype(x[s_start[i]:s_end[i], :] @ A_as_[h_in, r])
  *   empty or negative segments are skipped without reading w_ptrs[i]
  *   (sgmv_cutlass.cuh:39-44).  Rows at or beyond num_tokens are never accessed.
+ *   `scale` multiplies the fp32 sums before they are rounded (1 in every call of the reference's
+ *   legacy path; the `scaling` argument of lorax_server/utils/ops/sgmv_shrink.py:101-196).
  *
  * r must be a multiple of 8 in [8, 128]; h_in a multiple of 8; LORAX_A_RH with a rank that is not a
  * multiple of 16 additionally needs h_in to be a multiple of 128.  `tmp`/`tmp_bytes` is the caller's
@@ -157,8 +159,8 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
  */
 int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
-                      int32_t h_in, int32_t r, int32_t a_layout, int64_t layer_idx, void* tmp,
-                      int64_t tmp_bytes, int32_t dtype, void* stream);
+                      int32_t h_in, int32_t r, int32_t a_layout, int64_t layer_idx, float scale,
+                      void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
 
 /*
  * SGMV expand.  Replaces the expand direction of sgmv_cutlass (punica_ops.cc:338-367,
@@ -168,13 +170,16 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
  *     B = (dtype*)w_ptrs[i] + layer_idx * r * h_out                  // [r, h_out] (LORAX_B_RH)
  *     y[s:e, y_offset : y_offset + h_out] += dtype(v[s:e, :] @ B)    // row pitch y_stride
  *   With b_layout = LORAX_B_HR the stack holds B^T, [h_out, r] per layer, and the result is the same.
+ *   accumulate = 1 is the reference's only mode; accumulate = 0 stores dtype(v @ B) into the rows of the
+ *   segments instead of adding it (add_inputs=False of lorax_server/utils/ops/sgmv_expand.py:106-121).
  *
  * r must be a multiple of 8 in [8, 128]; h_out, y_offset and y_stride multiples of 8.
  */
 int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
                       int32_t h_out, int32_t b_layout, int64_t y_offset, int64_t y_stride,
-                      int64_t layer_idx, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
+                      int64_t layer_idx, int32_t accumulate, void* tmp, int64_t tmp_bytes,
+                      int32_t dtype, void* stream);
 
 /* Bytes of grouped-GEMM argument scratch for `num_problems` segments.  Replaces
  * sgmv_tmp_size (sgmv/sgmv_cutlass.cuh:54-58): 3 pointers + 3 int64 + one

@@ -64,14 +64,14 @@ _SIGNATURES = {
     "lorax_sgmv_shrink": (
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
-         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_void_p, _c.c_int64, _c.c_int32,
+         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_void_p, _c.c_int64, _c.c_int32,
          _c.c_void_p],
     ),
     "lorax_sgmv_expand": (
         _c.c_int,
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
-         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
-         _c.c_int32, _c.c_void_p],
+         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int32, _c.c_void_p,
+         _c.c_int64, _c.c_int32, _c.c_void_p],
     ),
     "lorax_sgmv_tmp_size": (_c.c_size_t, [_c.c_int32]),
     "lorax_init": (_c.c_int, [_c.c_int32]),
@@ -323,30 +323,30 @@ def _check_sgmv(y, x, w_ptr, s_start, s_end, tmp) -> None:
 
 
 def sgmv_expand(y, x, w_ptr, s_start, s_end, tmp, layer_idx, y_offset=0, y_slice_size=None,
-                transposed: bool = False) -> None:
+                transposed: bool = False, accumulate: bool = True) -> None:
     """lorax_sgmv_expand with an optional column window of y.  `transposed`: w_ptr addresses [L, h_out, r]
-    stacks (B^T) instead of the reference's [L, r, h_out]."""
+    stacks (B^T) instead of the reference's [L, r, h_out].  accumulate=False overwrites the segments' rows."""
     _check_sgmv(y, x, w_ptr, s_start, s_end, tmp)
     h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
     with torch.cuda.device(x.device):
         rc = lib().lorax_sgmv_expand(
             y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0),
             x.size(0), x.size(1), h_out, B_HR if transposed else B_RH, int(y_offset), y.size(1), int(layer_idx),
-            tmp.data_ptr(),
+            1 if accumulate else 0, tmp.data_ptr(),
             tmp.numel() * tmp.element_size(), _dtype_code(x), _stream(x),
         )
     if rc != 0:
         _raise_last(rc)
 
 
-def _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, a_layout) -> None:
+def _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, a_layout, scale: float = 1.0) -> None:
     _check_sgmv(y, x, w_ptr, s_start, s_end, tmp)
     if not torch.cuda.is_current_stream_capturing():
         init(x.device)
     with torch.cuda.device(x.device):
         rc = lib().lorax_sgmv_shrink(
             y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0),
-            x.size(0), x.size(1), y.size(1), a_layout, int(layer_idx), tmp.data_ptr(),
+            x.size(0), x.size(1), y.size(1), a_layout, int(layer_idx), float(scale), tmp.data_ptr(),
             tmp.numel() * tmp.element_size(), _dtype_code(x), _stream(x),
         )
     if rc != 0:
@@ -362,8 +362,9 @@ def sgmv_cutlass(y, x, w_ptr, s_start, s_end, tmp, layer_idx) -> None:
     return _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, A_HR)
 
 
-def sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx) -> None:
-    """dispatch_sgmv_shrink, punica_ops.cc:369-411: weights are [L, d_out, d_in], tmp is 8 MiB of uint8."""
+def sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, scale: float = 1.0) -> None:
+    """dispatch_sgmv_shrink, punica_ops.cc:369-411: weights are [L, d_out, d_in], tmp is 8 MiB of uint8.
+    `scale` (not in the reference's binding) multiplies the sums before they are rounded."""
     if isinstance(tmp, torch.Tensor) and tmp.dtype != torch.uint8:
         raise RuntimeError(f"CHECK_EQ(tmp.scalar_type(), at::ScalarType::Byte) failed. {tmp.dtype}")
-    return _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, A_RH)
+    return _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, A_RH, scale)

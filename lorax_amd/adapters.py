@@ -426,8 +426,9 @@ class LayerAdapterWeights:
 
 @dataclass
 class AdapterBatchData:
-    """adapters/weights.py:108-171. ``punica_wrapper`` and ``layer_to_lora_weights`` belong to the
-    reference's Triton path and are always None/empty here."""
+    """adapters/weights.py:108-171. ``punica_wrapper`` (lorax_amd.punica_wrapper.PunicaWrapper) and
+    ``layer_to_lora_weights`` (stack_preloaded_adapters) select the stacked-weight path of
+    LoraLinear.forward_layer_type, as in the reference; both are optional."""
 
     meta: AdapterBatchMetadata
     data: Dict[str, Dict[str, BatchAdapterWeights]]  # layer type -> adapter type -> batch data
@@ -480,3 +481,39 @@ class AdapterBatchData:
     @property
     def max_rank(self) -> int:
         return max(self.ranks(), default=0)
+
+
+def stack_preloaded_adapters(
+    layer_to_adapter_weights: Dict[str, LayerAdapterWeights],
+    adapter_indices: List[int],
+    device=None,
+) -> Dict[Tuple[str, int], Tuple[torch.Tensor, torch.Tensor]]:
+    """(layer type, layer) -> (lora_a_weights [num_adapters, r, h_in], lora_b_weights [num_adapters, h_out, r]) over
+    the given adapters in order, every adapter zero-padded to the largest rank of the stack (models/model.py:289-334).
+    Entry i of a stack belongs to adapter_indices[i]; PunicaWrapper.update_metadata maps adapter index k to entry
+    k - 1, so the caller numbers its preloaded adapters 1..n as the reference does."""
+    from lorax_amd.sgmv import pad_to_min_rank
+
+    out: Dict[Tuple[str, int], Tuple[torch.Tensor, torch.Tensor]] = {}
+    for layer_name, layer_adapter_weights in layer_to_adapter_weights.items():
+        per_layer_a: Dict[int, List[torch.Tensor]] = defaultdict(list)
+        per_layer_b: Dict[int, List[torch.Tensor]] = defaultdict(list)
+        for adapter_index in adapter_indices:
+            weights = _unwrap(layer_adapter_weights.adapter_weights.get(adapter_index))
+            if not isinstance(weights, LoraWeights):
+                continue
+            lora_a, lora_b = weights.weights_a_t, weights.weights_b_t  # [L, r, h_in], [L, h_out, r]
+            for layer_id in range(lora_a.size(0)):
+                per_layer_a[layer_id].append(lora_a[layer_id])
+                per_layer_b[layer_id].append(lora_b[layer_id])
+        for layer_id, a_list in per_layer_a.items():
+            b_list = per_layer_b[layer_id]
+            r = max(w.size(-1) for w in b_list)
+            a_list = [pad_to_min_rank(w, 0, r) for w in a_list]
+            b_list = [pad_to_min_rank(w, 1, r) for w in b_list]
+            lora_a = torch.stack(a_list).contiguous()
+            lora_b = torch.stack(b_list).contiguous()
+            if device is not None:
+                lora_a, lora_b = lora_a.to(device), lora_b.to(device)
+            out[(layer_name, layer_id)] = (lora_a, lora_b)
+    return out

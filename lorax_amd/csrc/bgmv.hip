@@ -198,7 +198,7 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
                                                  const typename D::E* __restrict__ B,
                                                  const int (&toks)[kGroup], int r, int h_out,
                                                  int col0, int64_t y_offset, int64_t y_stride,
-                                                 float scale) {
+                                                 float scale, bool accumulate_into_y) {
   using vec8 = typename D::vec8;
   using E = typename D::E;
   constexpr int kCols = kBgmvThreads / CP;  // columns per step of the workgroup
@@ -227,7 +227,7 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
 #pragma unroll
     for (int g = 0; g < NT; ++g) {
       yv[u][g] = static_cast<E>(0.f);
-      if (part == 0 && col[u] < h_out)
+      if (part == 0 && col[u] < h_out && accumulate_into_y)
         yv[u][g] = Y[static_cast<int64_t>(toks[g]) * y_stride + y_offset + col[u]];
     }
 #pragma unroll
@@ -250,7 +250,7 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
 
 template <typename D, int CP, int U>
 __device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const BatchSlot& slot, int num_tokens,
-                                                    int64_t layer_idx, float scale) {
+                                                    int64_t layer_idx, float scale, bool acc_y) {
   using E = typename D::E;
   const int h_out = P.width;
   const int r = P.narrow;
@@ -264,16 +264,16 @@ __device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const 
   const E* V = static_cast<const E*>(P.x);
   switch (n) {
     case 1:
-      bgmv_expand_body<D, CP, U, 1>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
+      bgmv_expand_body<D, CP, U, 1>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
       break;
     case 2:
-      bgmv_expand_body<D, CP, U, 2>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
+      bgmv_expand_body<D, CP, U, 2>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
       break;
     case 3:
-      bgmv_expand_body<D, CP, U, 3>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
+      bgmv_expand_body<D, CP, U, 3>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
       break;
     default:
-      bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale);
+      bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
       break;
   }
 }
@@ -287,24 +287,26 @@ __host__ __device__ __forceinline__ int expand_lanes_per_column(int r) {
 // One launch serves problems of different ranks: the workgroup picks the body for its problem's rank.
 template <typename D, int U>
 __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBatch batch, int count,
-                                                                   int num_tokens, int64_t layer_idx, float scale) {
+                                                                   int num_tokens, int64_t layer_idx, float scale,
+                                                                   int accumulate_into_y) {
+  const bool acc_y = accumulate_into_y != 0;
   const BatchSlot vb = batch_slot(batch, count);
   const BgmvProblem& P = batch.p[vb.problem];
   switch (expand_lanes_per_column(P.narrow)) {
     case 1:
-      bgmv_expand_problem<D, 1, U>(P, vb, num_tokens, layer_idx, scale);
+      bgmv_expand_problem<D, 1, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
     case 2:
-      bgmv_expand_problem<D, 2, U>(P, vb, num_tokens, layer_idx, scale);
+      bgmv_expand_problem<D, 2, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
     case 4:
-      bgmv_expand_problem<D, 4, U>(P, vb, num_tokens, layer_idx, scale);
+      bgmv_expand_problem<D, 4, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
     case 8:
-      bgmv_expand_problem<D, 8, U>(P, vb, num_tokens, layer_idx, scale);
+      bgmv_expand_problem<D, 8, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
     default:
-      bgmv_expand_problem<D, 16, U>(P, vb, num_tokens, layer_idx, scale);
+      bgmv_expand_problem<D, 16, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
   }
 }
@@ -616,7 +618,7 @@ static hipError_t launch_expand_u(BgmvArgs a, hipStream_t stream) {
   if (total == 0) return hipSuccess;
   if (total >= INT32_MAX) return hipErrorInvalidValue;
   hipLaunchKernelGGL((bgmv_expand_kernel<D, U>), dim3(static_cast<unsigned>(total)), dim3(kBgmvThreads), 0, stream,
-                     a.batch, a.count, static_cast<int>(a.num_tokens), a.layer_idx, a.scale);
+                     a.batch, a.count, static_cast<int>(a.num_tokens), a.layer_idx, a.scale, a.accumulate);
   return hipGetLastError();
 }
 

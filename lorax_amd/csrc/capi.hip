@@ -167,8 +167,8 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
   if (a.grid_rows == 0) return LORAX_OK;
   if (!a.expand && accumulate != 0 && accumulate != 1)
     return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
-  if (a.expand && accumulate != 1)
-    return fail(LORAX_EINVAL, "an expand launch always adds to y (accumulate must be 1)");
+  if (accumulate != 0 && accumulate != 1)
+    return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (num_tokens > 65535)
     return fail(LORAX_ENOKERNEL, "No suitable kernel. num_tokens=%lld exceeds 65535", (long long)num_tokens);
   const hipError_t e = launch_bgmv(a, static_cast<hipStream_t>(stream));
@@ -196,8 +196,8 @@ int lorax_bgmv_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems,
 
 int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
-                      int32_t h_in, int32_t r, int32_t a_layout, int64_t layer_idx, void* tmp,
-                      int64_t tmp_bytes, int32_t dtype, void* stream) {
+                      int32_t h_in, int32_t r, int32_t a_layout, int64_t layer_idx, float scale,
+                      void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
   if (num_segments < 0 || num_tokens < 0)
     return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments,
                 (long long)num_tokens);
@@ -241,6 +241,7 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
   a.a_layout = a_layout;
   a.layer_idx = layer_idx;
   a.dtype = dtype;
+  a.scale = scale;
   a.partials = ws.partials;
   a.partial_bytes = ws.partials ? kPartialBytes : 0;
   a.counters = ws.counters;
@@ -253,7 +254,10 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
 int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
                       int32_t h_out, int32_t b_layout, int64_t y_offset, int64_t y_stride,
-                      int64_t layer_idx, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
+                      int64_t layer_idx, int32_t accumulate, void* tmp, int64_t tmp_bytes, int32_t dtype,
+                      void* stream) {
+  if (accumulate != 0 && accumulate != 1)
+    return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (b_layout != LORAX_B_RH && b_layout != LORAX_B_HR) return fail(LORAX_EINVAL, "b_layout=%d", b_layout);
   if (num_segments < 0 || num_tokens < 0)
     return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments,
@@ -287,6 +291,7 @@ int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32
   a.layer_idx = layer_idx;
   a.dtype = dtype;
   a.a_layout = b_layout;
+  a.accumulate = accumulate;
   const hipError_t e = b_layout == LORAX_B_HR ? launch_sgmv_expand_t(a, static_cast<hipStream_t>(stream))
                                               : launch_sgmv_expand(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_expand launch failed: %s", hipGetErrorString(e));

@@ -76,6 +76,8 @@ struct SgmvArgs {
   int64_t y_stride;
   int64_t layer_idx;
   int dtype;
+  float scale;     // shrink: factor applied to the fp32 sums before rounding (1 in the reference's calls)
+  int accumulate;  // expand: 1 = add to y (the reference's only mode), 0 = overwrite the rows of the segments
   // library workspace of the current device (shrink split-K)
   float* partials;
   size_t partial_bytes;

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int r, int h_out,
     int64_t y_offset, int64_t y_stride, int64_t layer_idx, int rows_per_tile, int panels_per_wave,
-    int tile_slots) {
+    int tile_slots, int accumulate_into_y) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   const int lane = threadIdx.x & (kWave - 1);
@@ -110,6 +110,8 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
         const int row = rt.row0 + mb * 16 + c;
         const bool ok = live && row < rt.row_end;
         E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0;
+        y0 = keep_if<D>(accumulate_into_y != 0, y0);  // overwrite mode: the old y counts as zero
+        y1 = keep_if<D>(accumulate_into_y != 0, y1);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           y0[i] = accumulate<D>(y0[i], acc[0][i]);
@@ -156,7 +158,7 @@ static hipError_t launch_expand_t_ks(const SgmvArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((sgmv_expand_t_kernel<D, KS>), grid, dim3(kExpTThreads), 0, stream,
                      static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start,
                      a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.y_offset,
-                     a.y_stride, a.layer_idx, rows_per_tile, ppw, tile_slots);
+                     a.y_stride, a.layer_idx, rows_per_tile, ppw, tile_slots, a.accumulate);
   return hipGetLastError();
 }
 

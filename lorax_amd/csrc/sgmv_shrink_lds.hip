@@ -59,7 +59,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     typename D::E* __restrict__ V, const typename D::E* __restrict__ X,
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int r,
-    int64_t layer_idx, int stages) {
+    int64_t layer_idx, int stages, float scale) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   // NB = ceil(r / 16) rank blocks; the rank itself only needs to be a multiple of 8: rows of the A tile past
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
         }
         const int row = rt.row0 + (blk / NB) * 16 + (l & 15);
         const int col = (blk % NB) * 16 + 4 * (l >> 4);
-        if (row < rt.row_end && col < r) accumulate4<D>(V + static_cast<int64_t>(row) * r + col, sum);
+        if (row < rt.row_end && col < r) accumulate4<D>(V + static_cast<int64_t>(row) * r + col, sum * scale);
       }
     } else {
       // every wave owns its output blocks: no cross-wave reduction
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
 #pragma unroll
           for (int nb = 0; nb < NPW; ++nb) {
             const int col = (wn * NPW + nb) * 16 + 4 * g;
-            if (col < r) accumulate4<D>(V + static_cast<int64_t>(row) * r + col, acc[mb][nb]);
+            if (col < r) accumulate4<D>(V + static_cast<int64_t>(row) * r + col, acc[mb][nb] * scale);
           }
         }
       }
@@ -242,7 +242,7 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   dim3 grid(static_cast<unsigned>(tiles < (1 << 20) ? tiles : (1 << 20)));
   hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, static_cast<typename D::E*>(a.y),
                      static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end, a.num_segments,
-                     static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, stages);
+                     static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, stages, a.scale);
   return hipGetLastError();
 }
 

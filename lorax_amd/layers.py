@@ -84,6 +84,24 @@ class LoraLinear(nn.Module):
             data = self._lora_data(adapter_data, name)
             if data is None:
                 continue
+            # Stacked weights of preloaded adapters (utils/layers.py:79-105): one index into a
+            # [num_adapters, ...] stack per token instead of pointer tables per rank.
+            key = (name, self.layer_id)
+            wrapper = adapter_data.punica_wrapper
+            if (
+                wrapper is not None
+                and wrapper.enabled
+                and key in adapter_data.layer_to_lora_weights
+                and input.shape[0] <= wrapper.max_batch_size
+            ):
+                whole = end - start == result.shape[1]
+                lora_a_weights, lora_b_weights = adapter_data.layer_to_lora_weights[key]
+                wrapper.add_lora(
+                    result, input, lora_a_weights, lora_b_weights, 1.0,
+                    None if whole else start, None if whole else end - start,
+                    callback=self.collect_lora_a if tensor_parallel else None,
+                )
+                continue
             sliced = end - start != result.shape[1]
             for r, rs in data.rank_data.items():
                 if not data.use_sgmv:

@@ -242,3 +242,7 @@ def segmented_matmul(
     for wi, bi, s, e in zip(w, b, starts, ends):
         if e > s:
             y[s:e] = F.linear(x[s:e], wi, bi)
+
+
+# The stacked-weight front end of the reference lives in the same module there (punica.py:256-793).
+from lorax_amd.punica_wrapper import PunicaWrapper, compute_meta  # noqa: E402,F401

@@ -63,27 +63,27 @@ def test_bgmv_validation():
 def test_sgmv_shrink_validation():
     f = _native.lib().lorax_sgmv_shrink
     big = 8 * 1024 * 1024
-    assert f(P, P, P, P, P, 2, 16, 4096, 16, 0, 0, P, big - 1, 0, None) == ETMPSIZE and "8 * 1024 * 1024" in _err()
-    assert f(P, P, P, P, P, 2, 16, 4096, 8, 1, 0, P, 119, 0, None) == ETMPSIZE and "sgmv_tmp_size" in _err()
-    assert f(P, P, P, P, P, 0, 16, 4096, 16, 0, 0, P, big, 0, None) == OK  # no segments
-    assert f(P, P, P, P, P, 2, 16, 4096, 16, 7, 0, P, big, 0, None) == EINVAL  # layout
+    assert f(P, P, P, P, P, 2, 16, 4096, 16, 0, 0, 1.0, P, big - 1, 0, None) == ETMPSIZE and "8 * 1024 * 1024" in _err()
+    assert f(P, P, P, P, P, 2, 16, 4096, 8, 1, 0, 1.0, P, 119, 0, None) == ETMPSIZE and "sgmv_tmp_size" in _err()
+    assert f(P, P, P, P, P, 0, 16, 4096, 16, 0, 0, 1.0, P, big, 0, None) == OK  # no segments
+    assert f(P, P, P, P, P, 2, 16, 4096, 16, 7, 0, 1.0, P, big, 0, None) == EINVAL  # layout
     for r, h_in in ((8, 4104), (24, 4104), (144, 4096), (12, 4096)):
-        assert f(P, P, P, P, P, 2, 16, h_in, r, 0, 0, P, big, 0, None) == ENOKERNEL, r
-    assert f(P, P, P, P, P, 2, 16, 4100, 16, 0, 0, P, big, 0, None) == ENOKERNEL
-    assert f(P, P, P, None, P, 2, 16, 4096, 16, 0, 0, P, big, 0, None) == EINVAL
-    assert f(P, P, P, P, P, 2, 16, 4096, 16, 0, 0, P, big, 5, None) == ENOKERNEL  # dtype
+        assert f(P, P, P, P, P, 2, 16, h_in, r, 0, 0, 1.0, P, big, 0, None) == ENOKERNEL, r
+    assert f(P, P, P, P, P, 2, 16, 4100, 16, 0, 0, 1.0, P, big, 0, None) == ENOKERNEL
+    assert f(P, P, P, None, P, 2, 16, 4096, 16, 0, 0, 1.0, P, big, 0, None) == EINVAL
+    assert f(P, P, P, P, P, 2, 16, 4096, 16, 0, 0, 1.0, P, big, 5, None) == ENOKERNEL  # dtype
 
 
 def test_sgmv_expand_validation():
     f = _native.lib().lorax_sgmv_expand
     for layout in (_native.B_RH, _native.B_HR):
-        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 0, 4096, 0, P, 121, 1, None) == ETMPSIZE
-        assert f(P, P, P, P, P, 0, 16, 16, 4096, layout, 0, 4096, 0, None, 0, 1, None) == OK
+        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 0, 4096, 0, 1, P, 121, 1, None) == ETMPSIZE
+        assert f(P, P, P, P, P, 0, 16, 16, 4096, layout, 0, 4096, 0, 1, None, 0, 1, None) == OK
         for r, h in [(4, 4096), (136, 4096), (16, 4100)]:
-            assert f(P, P, P, P, P, 2, 16, r, h, layout, 0, h, 0, P, 120, 1, None) == ENOKERNEL, (r, h)
-        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 4, 8192, 0, P, 120, 1, None) == EINVAL  # unaligned window
-        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 4096, 4096, 0, P, 120, 1, None) == EINVAL  # too wide
-    assert f(P, P, P, P, P, 2, 16, 16, 4096, 2, 0, 4096, 0, P, 120, 1, None) == EINVAL  # unknown layout
+            assert f(P, P, P, P, P, 2, 16, r, h, layout, 0, h, 0, 1, P, 120, 1, None) == ENOKERNEL, (r, h)
+        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 4, 8192, 0, 1, P, 120, 1, None) == EINVAL  # unaligned window
+        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 4096, 4096, 0, 1, P, 120, 1, None) == EINVAL  # too wide
+    assert f(P, P, P, P, P, 2, 16, 16, 4096, 2, 0, 4096, 0, 1, P, 120, 1, None) == EINVAL  # unknown layout
 
 
 def test_python_binding_rejects_cpu_tensors():
