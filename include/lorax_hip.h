@@ -35,6 +35,7 @@ extern "C" {
 #define LORAX_ENOKERNEL 2  /* shape outside what the kernels cover ("No suitable kernel.") */
 #define LORAX_ELAUNCH 3    /* the HIP runtime refused the launch                            */
 #define LORAX_ETMPSIZE 4   /* tmp buffer size does not match the reference's contract       */
+#define LORAX_ESPACE 5     /* an output buffer of the caller is too small; sizes are reported */
 
 #define LORAX_F16 0
 #define LORAX_BF16 1
@@ -185,6 +186,51 @@ int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32
  * sgmv_tmp_size (sgmv/sgmv_cutlass.cuh:54-58): 3 pointers + 3 int64 + one
  * 3 x int32 problem size per segment = 60 * num_problems. */
 size_t lorax_sgmv_tmp_size(int32_t num_problems);
+
+/*
+ * Routing tables of one batch for ALL layer types, built on the host into one packed buffer (one
+ * host-to-device copy).  Replaces, per step, find_segments (lorax_server/utils/segments.py:6-34) and
+ * the table building of BatchLoraWeights.load for every layer type (lorax_server/adapters/lora.py:
+ * 290-396: grouping of segments by rank, pointer tables, segment bounds, per-token indices), and adds the
+ * routing plan of lorax_bgmv_multi / lorax_bgmv_lora_multi.  Runs on the CPU; touches no GPU state.
+ *
+ * adapter_indices[num_tokens]: adapter of every token (any value; tokens of adapters without an entry
+ *   are not routed).  entries: for layer type 0, 1, ... the adapters that have weights for it
+ *   (entry_counts[t] of them, sorted by `adapter`), with the device addresses of their resident stacks.
+ * Outputs: segment_bounds[num_tokens + 1] / segment_owners[num_tokens] (first *num_segments + 1 / *num_segments
+ *   used); `groups`: one descriptor per (layer type, rank), ranks in order of first appearance, with byte
+ *   offsets into `packed`.  Returns LORAX_ESPACE when `packed` or `groups` is too small (or NULL), with
+ *   *packed_bytes and *num_groups set to what is needed.
+ */
+typedef struct lorax_adapter_entry {
+  int64_t adapter; /* adapter index as it appears in adapter_indices            */
+  int64_t a_addr;  /* device address of the [L, r, h_in] stack                   */
+  int64_t b_addr;  /* device address of the [L, h_out, r] stack                  */
+  int32_t rank;
+  int32_t reserved;
+} lorax_adapter_entry_t;
+
+typedef struct lorax_table_group {
+  int32_t layer_type;   /* index into entry_counts                                       */
+  int32_t rank;
+  int32_t use_sgmv;     /* 1: segment tables (prefill, or a rank above 128); 0: per-token */
+  int32_t num_segments; /* entries of the group's pointer tables                          */
+  int32_t num_chunks;   /* routing-plan records (use_sgmv = 0)                            */
+  int32_t reserved;
+  int64_t a_ptr_off;    /* int64[num_segments] stack addresses per segment                */
+  int64_t b_ptr_off;
+  int64_t starts_off;   /* int32[num_segments] (use_sgmv = 1), else -1                    */
+  int64_t ends_off;
+  int64_t indices_off;  /* int64[num_tokens] slot in the group's tables or -1 (use_sgmv = 0) */
+  int64_t plan_off;     /* int64[num_chunks][8] routing plan (use_sgmv = 0)               */
+} lorax_table_group_t;
+
+int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t num_tokens,
+                             const lorax_adapter_entry_t* entries, const int32_t* entry_counts,
+                             int32_t num_layer_types, int32_t prefill, int32_t* segment_bounds,
+                             int64_t* segment_owners, int32_t* num_segments, void* packed,
+                             int64_t packed_capacity, int64_t* packed_bytes, lorax_table_group_t* groups,
+                             int32_t group_capacity, int32_t* num_groups);
 
 /*
  * Allocates (once per device, idempotent) the library's workspace on `device`:

@@ -42,6 +42,22 @@ class BgmvProblem(ctypes.Structure):
     ]
 
 
+class AdapterEntry(ctypes.Structure):
+    """lorax_adapter_entry_t of include/lorax_hip.h."""
+
+    _fields_ = [("adapter", _c.c_int64), ("a_addr", _c.c_int64), ("b_addr", _c.c_int64), ("rank", _c.c_int32),
+                ("reserved", _c.c_int32)]
+
+
+class TableGroup(ctypes.Structure):
+    """lorax_table_group_t of include/lorax_hip.h."""
+
+    _fields_ = [("layer_type", _c.c_int32), ("rank", _c.c_int32), ("use_sgmv", _c.c_int32),
+                ("num_segments", _c.c_int32), ("num_chunks", _c.c_int32), ("reserved", _c.c_int32),
+                ("a_ptr_off", _c.c_int64), ("b_ptr_off", _c.c_int64), ("starts_off", _c.c_int64),
+                ("ends_off", _c.c_int64), ("indices_off", _c.c_int64), ("plan_off", _c.c_int64)]
+
+
 MAX_BGMV_PROBLEMS = 16
 MAX_FUSED_BGMV_PROBLEMS = 4
 
@@ -74,6 +90,12 @@ _SIGNATURES = {
          _c.c_int64, _c.c_int32, _c.c_void_p],
     ),
     "lorax_sgmv_tmp_size": (_c.c_size_t, [_c.c_int32]),
+    "lorax_build_batch_tables": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int32, _c.c_void_p, _c.c_void_p,
+         _c.POINTER(_c.c_int32), _c.c_void_p, _c.c_int64, _c.POINTER(_c.c_int64), _c.POINTER(TableGroup), _c.c_int32,
+         _c.POINTER(_c.c_int32)],
+    ),
     "lorax_init": (_c.c_int, [_c.c_int32]),
     "lorax_workspace_bytes": (_c.c_size_t, []),
     "lorax_last_error": (_c.c_char_p, []),
@@ -368,3 +390,38 @@ def sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, scale: float = 1.0)
     if isinstance(tmp, torch.Tensor) and tmp.dtype != torch.uint8:
         raise RuntimeError(f"CHECK_EQ(tmp.scalar_type(), at::ScalarType::Byte) failed. {tmp.dtype}")
     return _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, A_RH, scale)
+
+
+ESPACE = 5
+ENTRY_DTYPE = [("adapter", "<i8"), ("a_addr", "<i8"), ("b_addr", "<i8"), ("rank", "<i4"), ("reserved", "<i4")]
+
+
+def build_batch_tables(adapter_indices, entries, entry_counts, prefill: bool):
+    """lorax_build_batch_tables on numpy arrays: adapter_indices int64 [T]; entries a structured array of
+    ENTRY_DTYPE, the layer types' adapters one after the other, each type sorted by adapter; entry_counts int32
+    per type.  Returns (segment bounds int32 [S+1], segment owners int64 [S], packed uint8 buffer, groups)."""
+    import numpy as np
+
+    adapter_indices = np.ascontiguousarray(adapter_indices, dtype=np.int64)
+    entries = np.ascontiguousarray(entries, dtype=ENTRY_DTYPE)
+    entry_counts = np.ascontiguousarray(entry_counts, dtype=np.int32)
+    T = adapter_indices.shape[0]
+    bounds = np.zeros(T + 1, dtype=np.int32)
+    owners = np.zeros(max(T, 1), dtype=np.int64)
+    nseg, ngroups, nbytes = _c.c_int32(0), _c.c_int32(0), _c.c_int64(0)
+    capacity, group_capacity = 64 * 1024, 64
+    while True:
+        packed = np.zeros(capacity, dtype=np.uint8)
+        groups = (TableGroup * group_capacity)()
+        rc = lib().lorax_build_batch_tables(
+            adapter_indices.ctypes.data, T, entries.ctypes.data, entry_counts.ctypes.data, entry_counts.shape[0],
+            1 if prefill else 0, bounds.ctypes.data, owners.ctypes.data, ctypes.byref(nseg), packed.ctypes.data,
+            capacity, ctypes.byref(nbytes), groups, group_capacity, ctypes.byref(ngroups),
+        )
+        if rc == ESPACE:
+            capacity = max(capacity, int(nbytes.value))
+            group_capacity = max(group_capacity, int(ngroups.value))
+            continue
+        if rc != 0:
+            _raise_last(rc)
+        return bounds[: nseg.value + 1], owners[: nseg.value], packed[: nbytes.value], list(groups[: ngroups.value])

@@ -391,12 +391,33 @@ class LayerAdapterWeights:
 
     def __init__(self):
         self.adapter_weights: Dict[int, AdapterWeights] = {}
+        self._lora_entries = None  # cached argument of the native table builder
 
     def add_adapter(self, adapter_idx: int, weights: AdapterWeights):
         self.adapter_weights[adapter_idx] = weights
+        self._lora_entries = None
 
     def remove_adapter(self, adapter_idx: int):
         self.adapter_weights.pop(adapter_idx, None)
+        self._lora_entries = None
+
+    def lora_entries(self):
+        """(adapter, address of the [L, r, h_in] stack, address of the [L, h_out, r] stack, rank) of every LoRA
+        adapter of the layer type, sorted by adapter, as a numpy array of _native.ENTRY_DTYPE; None if an adapter
+        of another kind is loaded.  Rebuilt only when adapters come or go."""
+        if self._lora_entries is None:
+            import numpy as np
+
+            from lorax_amd import _native
+
+            rows = []
+            for idx in sorted(self.adapter_weights):
+                w = _unwrap(self.adapter_weights[idx])
+                if not isinstance(w, LoraWeights) or w.get_batch_types() != [BatchLoraWeights]:
+                    return None
+                rows.append((idx, w.weights_a_t.data_ptr(), w.weights_b_t.data_ptr(), w.lora_a_r, 0))
+            self._lora_entries = np.array(rows, dtype=_native.ENTRY_DTYPE)
+        return self._lora_entries
 
     @property
     def max_speculative_tokens(self) -> int:
@@ -445,14 +466,16 @@ class AdapterBatchData:
         prefill: bool = False,
         prefill_head_indices: Optional[torch.Tensor] = None,
     ) -> "AdapterBatchData":
-        data = {}
-        for layer_name, layer_weights in weights.items():
-            if layer_weights.is_empty():
-                continue
-            head = prefill_head_indices if layer_name == LM_HEAD else None
-            batched = layer_weights.get_data(meta, layer_name, prefill, head)
-            if batched:
-                data[layer_name] = batched
+        data = _native_batch_tables(meta, weights, prefill) if prefill_head_indices is None else None
+        if data is None:
+            data = {}
+            for layer_name, layer_weights in weights.items():
+                if layer_weights.is_empty():
+                    continue
+                head = prefill_head_indices if layer_name == LM_HEAD else None
+                batched = layer_weights.get_data(meta, layer_name, prefill, head)
+                if batched:
+                    data[layer_name] = batched
         return AdapterBatchData(
             meta=meta,
             data=data,
@@ -517,3 +540,90 @@ def stack_preloaded_adapters(
                 lora_a, lora_b = lora_a.to(device), lora_b.to(device)
             out[(layer_name, layer_id)] = (lora_a, lora_b)
     return out
+
+
+def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAdapterWeights],
+                         prefill: bool) -> Optional[Dict[str, Dict[str, BatchAdapterWeights]]]:
+    """The tables of BatchLoraWeights.load for every layer type from one call of the native builder and one
+    host-to-device copy.  None (the caller then takes the per-layer-type Python path) when the library is not
+    loaded or a layer type holds adapters that are not plain LoRA."""
+    from lorax_amd import _native
+
+    if not _native.available():
+        return None
+    import numpy as np
+
+    names = [n for n, lw in weights.items() if not lw.is_empty()]
+    tables = [weights[n].lora_entries() for n in names]
+    if not names or any(t is None for t in tables):
+        return None
+    device = meta.adapter_indices.device
+    indices = meta.adapter_indices.detach().cpu().numpy()
+    bounds, owners, packed, groups = _native.build_batch_tables(
+        indices, np.concatenate(tables), np.array([len(t) for t in tables], dtype=np.int32), prefill
+    )
+    dev = torch.from_numpy(packed).to(device)
+    dev64, dev32 = dev.view(torch.int64), dev.view(torch.int32)
+    seg_adapters = owners.tolist()
+    T = int(indices.shape[0])
+
+    by_type: Dict[int, List] = defaultdict(list)
+    for g in groups:
+        by_type[g.layer_type].append(g)
+    data: Dict[str, Dict[str, BatchAdapterWeights]] = {}
+    for lt, type_groups in by_type.items():
+        layer_name = names[lt]
+        layer = weights[layer_name]
+        loras = {a: _unwrap(layer.adapter_weights[a]) for a in set(seg_adapters) if a in layer.adapter_weights}
+        use_sgmv = bool(type_groups[0].use_sgmv)
+        null = EMPTY_TENSOR.data_ptr()
+
+        def table(layout: str, loras=loras) -> torch.Tensor:
+            addr = [getattr(loras[i], layout).data_ptr() if i in loras else null for i in seg_adapters]
+            return torch.tensor(addr, dtype=torch.int64, device=device)
+
+        rank_data: Dict[int, RankSegments] = {}
+        for g in type_groups:
+            n = g.num_segments
+            a_ptr = dev64[g.a_ptr_off // 8 : g.a_ptr_off // 8 + n]
+            b_ptr = dev64[g.b_ptr_off // 8 : g.b_ptr_off // 8 + n]
+            if use_sgmv:
+                tmp_shrink, tmp_expand = get_tmp_tensors(n, g.rank, device)
+                segs = [s for s, a in enumerate(seg_adapters) if a in loras and loras[a].lora_a_r == g.rank]
+                rank_data[g.rank] = RankSegments(
+                    rank=g.rank,
+                    lora_a_ptr=(lambda segs=segs, table=table: table("weights_a")[segs]),
+                    lora_b_ptr=(lambda segs=segs, table=table: table("weights_b")[segs]),
+                    tmp_shrink=tmp_shrink,
+                    tmp_expand=tmp_expand,
+                    segment_starts=dev32[g.starts_off // 4 : g.starts_off // 4 + n],
+                    segment_ends=dev32[g.ends_off // 4 : g.ends_off // 4 + n],
+                    indices=None,
+                    lora_a_t_ptr=a_ptr,
+                    lora_b_t_ptr=b_ptr,
+                )
+            else:
+                rank_data[g.rank] = RankSegments(
+                    rank=g.rank,
+                    lora_a_ptr=a_ptr,
+                    lora_b_ptr=b_ptr,
+                    tmp_shrink=None,
+                    tmp_expand=None,
+                    segment_starts=None,
+                    segment_ends=None,
+                    indices=dev64[g.indices_off // 8 : g.indices_off // 8 + T],
+                    plan=dev64[g.plan_off // 8 : g.plan_off // 8 + g.num_chunks * BGMV_PLAN_WORDS].view(
+                        g.num_chunks, BGMV_PLAN_WORDS),
+                )
+        data[layer_name] = {
+            LORA: BatchLoraWeights(
+                lora_a=_LayoutView(loras, "weights_a"),
+                lora_b=_LayoutView(loras, "weights_b"),
+                adapter_index_configs={a: lw.adapter_config for a, lw in loras.items()},
+                rank_data=rank_data,
+                use_sgmv=use_sgmv,
+                layer_name=layer_name,
+                prefill_head_indices=None,
+            )
+        }
+    return data

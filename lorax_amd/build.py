@@ -14,7 +14,8 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "liblorax_hip.so"
-SOURCES = ["capi.hip", "bgmv.hip", "sgmv_shrink.hip", "sgmv_shrink_lds.hip", "sgmv_expand.hip", "sgmv_expand_t.hip"]
+SOURCES = ["capi.hip", "bgmv.hip", "sgmv_shrink.hip", "sgmv_shrink_lds.hip", "sgmv_expand.hip", "sgmv_expand_t.hip",
+           "batch_tables.hip"]
 ARCH = "gfx950"
 
 # -packed-fp32-ops is switched off on purpose: the packed fp32 forms hipcc would

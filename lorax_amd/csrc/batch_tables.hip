@@ -1,0 +1,189 @@
+// Host-side builder of the per-batch routing tables - no device code in this file.
+//
+// Restates, for all layer types of a batch at once, what the reference computes per layer type and per
+// step in Python: find_segments (lorax_server/utils/segments.py:6-34), the grouping of segments by LoRA
+// rank and the per-group pointer tables, segment bounds and per-token indices of BatchLoraWeights.load
+// (lorax_server/adapters/lora.py:253-396), plus the routing plan of the batched BGMV launches.  Everything
+// goes into ONE packed buffer that the caller uploads with a single host-to-device copy; the reference
+// issues several small copies per layer type and rank.
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+#include "kernels.h"
+
+namespace {
+
+constexpr int kPlanGroup = 4;   // tokens per routing-plan record
+constexpr int kBgmvMaxRank = 128;  // BGMV_MAX_RANK, lorax_server/utils/punica.py:39
+
+struct Packer {
+  char* base;
+  int64_t capacity;
+  int64_t used = 0;
+  // Reserves `bytes` (16-byte aligned); returns the offset.  Keeps counting past the capacity so that the
+  // caller learns the size it needs.
+  int64_t reserve(int64_t bytes) {
+    const int64_t off = used;
+    used += (bytes + 15) / 16 * 16;
+    return off;
+  }
+  template <typename T>
+  T* at(int64_t off) { return used <= capacity ? reinterpret_cast<T*>(base + off) : nullptr; }
+};
+
+const lorax_adapter_entry_t* find_entry(const lorax_adapter_entry_t* first, int32_t count, int64_t adapter) {
+  const lorax_adapter_entry_t* last = first + count;
+  const lorax_adapter_entry_t* it =
+      std::lower_bound(first, last, adapter, [](const lorax_adapter_entry_t& e, int64_t a) { return e.adapter < a; });
+  return (it != last && it->adapter == adapter) ? it : nullptr;
+}
+
+}  // namespace
+
+extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t num_tokens,
+                                        const lorax_adapter_entry_t* entries, const int32_t* entry_counts,
+                                        int32_t num_layer_types, int32_t prefill, int32_t* segment_bounds,
+                                        int64_t* segment_owners, int32_t* num_segments_out, void* packed,
+                                        int64_t packed_capacity, int64_t* packed_bytes, lorax_table_group_t* groups,
+                                        int32_t group_capacity, int32_t* num_groups_out) {
+  if (num_tokens < 0 || num_layer_types < 0 || (num_tokens > 0 && adapter_indices == nullptr) ||
+      segment_bounds == nullptr || segment_owners == nullptr || num_segments_out == nullptr ||
+      packed_bytes == nullptr || num_groups_out == nullptr || (num_layer_types > 0 && entry_counts == nullptr))
+    return LORAX_EINVAL;
+
+  // Runs of equal adapter index (segments.py:6-34): bounds[0] = 0, a bound at every change, bounds[S] = T.
+  int32_t num_segments = 0;
+  segment_bounds[0] = 0;
+  for (int64_t t = 0; t < num_tokens; ++t) {
+    if (t == 0 || adapter_indices[t] != adapter_indices[t - 1]) {
+      segment_bounds[num_segments] = static_cast<int32_t>(t);
+      segment_owners[num_segments] = adapter_indices[t];
+      ++num_segments;
+    }
+  }
+  segment_bounds[num_segments] = static_cast<int32_t>(num_tokens);
+  *num_segments_out = num_segments;
+
+  Packer pack{static_cast<char*>(packed), packed != nullptr ? packed_capacity : 0};
+  int32_t num_groups = 0;
+  std::vector<const lorax_adapter_entry_t*> seg_entry(num_segments);
+  std::vector<int32_t> group_of_rank;          // ranks in order of first appearance
+  std::vector<std::vector<int32_t>> group_segs;  // segments of each rank group
+  std::vector<int32_t> slot_of_seg(num_segments);
+  std::vector<int32_t> token_seg(num_tokens);
+  for (int32_t s = 0; s < num_segments; ++s)
+    for (int32_t t = segment_bounds[s]; t < segment_bounds[s + 1]; ++t) token_seg[t] = s;
+
+  const lorax_adapter_entry_t* type_entries = entries;
+  for (int32_t lt = 0; lt < num_layer_types; ++lt) {
+    const int32_t count = entry_counts[lt];
+    // segments covered by an adapter that has weights for this layer type
+    int max_rank = 0;
+    bool any = false;
+    for (int32_t s = 0; s < num_segments; ++s) {
+      seg_entry[s] = count > 0 ? find_entry(type_entries, count, segment_owners[s]) : nullptr;
+      if (seg_entry[s] != nullptr) {
+        any = true;
+        max_rank = std::max(max_rank, static_cast<int>(seg_entry[s]->rank));
+      }
+    }
+    type_entries += count;
+    if (!any) continue;
+    const bool use_sgmv = prefill != 0 || max_rank > kBgmvMaxRank;  // lora.py:311
+
+    group_of_rank.clear();
+    group_segs.clear();
+    for (int32_t s = 0; s < num_segments; ++s) {
+      if (seg_entry[s] == nullptr) continue;
+      const int32_t rank = seg_entry[s]->rank;
+      size_t g = 0;
+      while (g < group_of_rank.size() && group_of_rank[g] != rank) ++g;
+      if (g == group_of_rank.size()) {
+        group_of_rank.push_back(rank);
+        group_segs.emplace_back();
+      }
+      group_segs[g].push_back(s);
+    }
+
+    for (size_t g = 0; g < group_of_rank.size(); ++g) {
+      const std::vector<int32_t>& segs = group_segs[g];
+      const int32_t n = static_cast<int32_t>(segs.size());
+      lorax_table_group_t desc{};
+      desc.layer_type = lt;
+      desc.rank = group_of_rank[g];
+      desc.use_sgmv = use_sgmv ? 1 : 0;
+      desc.num_segments = n;
+      desc.a_ptr_off = pack.reserve(static_cast<int64_t>(n) * 8);
+      desc.b_ptr_off = pack.reserve(static_cast<int64_t>(n) * 8);
+      if (int64_t* a = pack.at<int64_t>(desc.a_ptr_off)) {
+        int64_t* b = pack.at<int64_t>(desc.b_ptr_off);
+        for (int32_t i = 0; i < n; ++i) {
+          a[i] = seg_entry[segs[i]]->a_addr;
+          b[i] = seg_entry[segs[i]]->b_addr;
+        }
+      }
+      desc.starts_off = desc.ends_off = desc.indices_off = desc.plan_off = -1;
+      if (use_sgmv) {
+        desc.starts_off = pack.reserve(static_cast<int64_t>(n) * 4);
+        desc.ends_off = pack.reserve(static_cast<int64_t>(n) * 4);
+        if (int32_t* st = pack.at<int32_t>(desc.starts_off)) {
+          int32_t* en = pack.at<int32_t>(desc.ends_off);
+          for (int32_t i = 0; i < n; ++i) {
+            st[i] = segment_bounds[segs[i]];
+            en[i] = segment_bounds[segs[i] + 1];
+          }
+        }
+      } else {
+        // slot of a token = position of the FIRST segment of its adapter inside this group's pointer slice
+        // (lora.py:354-366); tokens of other ranks, of adapters without weights here and of no adapter: -1.
+        std::fill(slot_of_seg.begin(), slot_of_seg.end(), -1);
+        for (int32_t i = 0; i < n; ++i) {
+          int32_t first = i;
+          for (int32_t j = 0; j < i; ++j)
+            if (segment_owners[segs[j]] == segment_owners[segs[i]]) { first = j; break; }
+          slot_of_seg[segs[i]] = first;
+        }
+        desc.indices_off = pack.reserve(num_tokens * 8);
+        int64_t* idx = pack.at<int64_t>(desc.indices_off);
+        // chunks: tokens of one slot, in token order, cut into groups of kPlanGroup; slots in order of their
+        // first token
+        std::vector<std::vector<int32_t>> toks_of_slot(n);
+        std::vector<int32_t> slot_order;
+        for (int64_t t = 0; t < num_tokens; ++t) {
+          const int32_t slot = slot_of_seg[token_seg[t]];
+          if (idx != nullptr) idx[t] = slot;
+          if (slot >= 0) {
+            if (toks_of_slot[slot].empty()) slot_order.push_back(slot);
+            toks_of_slot[slot].push_back(static_cast<int32_t>(t));
+          }
+        }
+        int32_t chunks = 0;
+        for (int32_t slot : slot_order) chunks += (static_cast<int32_t>(toks_of_slot[slot].size()) + kPlanGroup - 1) / kPlanGroup;
+        desc.num_chunks = chunks;
+        desc.plan_off = pack.reserve(static_cast<int64_t>(chunks) * lorax::kPlanRecordWords * 8);
+        if (int64_t* rec = pack.at<int64_t>(desc.plan_off)) {
+          for (int32_t slot : slot_order) {
+            const std::vector<int32_t>& toks = toks_of_slot[slot];
+            for (size_t i = 0; i < toks.size(); i += kPlanGroup) {
+              const int cnt = static_cast<int>(std::min<size_t>(kPlanGroup, toks.size() - i));
+              rec[0] = cnt;
+              for (int q = 0; q < kPlanGroup; ++q) rec[1 + q] = toks[q < cnt ? i + q : i];
+              rec[5] = seg_entry[segs[slot]]->a_addr;
+              rec[6] = seg_entry[segs[slot]]->b_addr;
+              rec[7] = 0;
+              rec += lorax::kPlanRecordWords;
+            }
+          }
+        }
+      }
+      if (groups != nullptr && num_groups < group_capacity) groups[num_groups] = desc;
+      ++num_groups;
+    }
+  }
+  *packed_bytes = pack.used;
+  *num_groups_out = num_groups;
+  if (pack.used > pack.capacity || num_groups > group_capacity || (groups == nullptr && num_groups > 0))
+    return LORAX_ESPACE;
+  return LORAX_OK;
+}

@@ -305,3 +305,74 @@ def test_prefill_tables_touch_only_resident_layouts():
     assert lws[0].weights_a.shape == (L, h, 8) and lws[0].weights_a_t.shape == (L, 8, h)
     assert data.lora_b[1].shape == (L, 16, h) and lws[1]._weights_b is not None
     assert torch.equal(lws[0].weights_a.transpose(1, 2), lws[0].weights_a_t)
+
+
+@pytest.mark.parametrize("config", [1, 2, 3, 4, 5])
+def test_native_table_builder_matches_python_tables(config):
+    """lorax_build_batch_tables (one call, one packed buffer for all layer types) against the per-layer-type Python
+    restatement of BatchLoraWeights.load, which the golden vectors of the reference's test_lora.py pin."""
+    from lorax_amd import synthetic
+    from lorax_amd.adapters import LORA, AdapterBatchData
+    from lorax_amd.segments import find_segments
+
+    kwargs = {"num_layers": 1}
+    if config in (3,):
+        kwargs.update(num_segments=12, max_len=40)
+    if config == 4:
+        kwargs.update(num_tokens=96, num_adapters=40)
+    if config == 5:
+        kwargs.update(prefill_tokens=50, decode_tokens=24, num_adapters=12)
+    w = synthetic.CONFIGS[config]("cpu", **kwargs)
+    fast = AdapterBatchData.from_meta(w.meta, w.weights, prefill=w.prefill)
+    assert set(fast.data) == {n for n, lw in w.weights.items() if not lw.is_empty()}
+    for name, layer in w.weights.items():
+        slow = layer.get_data(w.meta, name, w.prefill, None)
+        if not slow:
+            assert name not in fast.data
+            continue
+        a, b = fast.data[name][LORA], slow[LORA]
+        assert a.use_sgmv == b.use_sgmv and a.layer_name == b.layer_name
+        assert list(a.rank_data) == list(b.rank_data)  # ranks in order of first appearance
+        assert a.adapter_index_configs.keys() == b.adapter_index_configs.keys()
+        for rank in a.rank_data:
+            ra, rb = a.rank_data[rank], b.rank_data[rank]
+            for field in ("lora_a_t_ptr", "lora_b_t_ptr", "segment_starts", "segment_ends", "indices", "plan"):
+                ta, tb = getattr(ra, field), getattr(rb, field)
+                assert (ta is None) == (tb is None), field
+                if ta is not None:
+                    assert ta.dtype == tb.dtype and torch.equal(ta, tb), (name, rank, field)
+            assert torch.equal(ra.lora_a_ptr, rb.lora_a_ptr) and torch.equal(ra.lora_b_ptr, rb.lora_b_ptr)
+    bounds, owners = find_segments(w.meta.adapter_indices)
+    assert w.meta.adapter_segments.tolist() == bounds and w.meta.segment_indices == owners
+
+
+def test_native_table_builder_reports_the_space_it_needs():
+    import ctypes
+
+    import numpy as np
+
+    from lorax_amd import _native
+
+    idx = np.array([3, 3, 7, -1, 3], dtype=np.int64)
+    entries = np.array([(3, 1000, 2000, 8, 0), (7, 3000, 4000, 16, 0)], dtype=_native.ENTRY_DTYPE)
+    counts = np.array([2], dtype=np.int32)
+    bounds, owners = np.zeros(6, dtype=np.int32), np.zeros(5, dtype=np.int64)
+    nseg, ngroups, nbytes = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int64()
+    f = _native.lib().lorax_build_batch_tables
+    rc = f(idx.ctypes.data, 5, entries.ctypes.data, counts.ctypes.data, 1, 0, bounds.ctypes.data, owners.ctypes.data,
+           ctypes.byref(nseg), None, 0, ctypes.byref(nbytes), None, 0, ctypes.byref(ngroups))
+    assert rc == _native.ESPACE and ngroups.value == 2 and nbytes.value > 0
+    assert bounds[: nseg.value + 1].tolist() == [0, 2, 3, 4, 5] and owners[: nseg.value].tolist() == [3, 7, -1, 3]
+    b, o, packed, groups = _native.build_batch_tables(idx, entries, counts, prefill=False)
+    assert packed.nbytes == nbytes.value and [g.rank for g in groups] == [8, 16]
+    g8 = groups[0]
+    plan = packed.view(np.int64)[g8.plan_off // 8 : g8.plan_off // 8 + 8 * g8.num_chunks].reshape(-1, 8)
+    assert plan.tolist() == [[3, 0, 1, 4, 0, 1000, 2000, 0]]  # adapter 3's tokens, both runs in one chunk
+    indices = packed.view(np.int64)[g8.indices_off // 8 : g8.indices_off // 8 + 5]
+    assert indices.tolist() == [0, 0, -1, -1, 0]
+    # prefill: segment tables instead
+    _, _, packed, groups = _native.build_batch_tables(idx, entries, counts, prefill=True)
+    g8 = groups[0]
+    assert g8.use_sgmv == 1 and g8.num_segments == 2 and g8.plan_off == -1
+    assert packed.view(np.int32)[g8.starts_off // 4 : g8.starts_off // 4 + 2].tolist() == [0, 4]
+    assert packed.view(np.int32)[g8.ends_off // 4 : g8.ends_off // 4 + 2].tolist() == [2, 5]
