@@ -154,7 +154,7 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
  *   legacy path; the `scaling` argument of lorax_server/utils/ops/sgmv_shrink.py:101-196).
  *
  * r must be a multiple of 8 in [8, 128]; h_in a multiple of 8; LORAX_A_RH with a rank that is not a
- * multiple of 16 additionally needs h_in to be a multiple of 128.  `tmp`/`tmp_bytes` is the caller's
+ * multiple of 16 additionally needs h_in to be a multiple of 128 or num_tokens <= 512.  `tmp`/`tmp_bytes` is the caller's
  * scratch and is only validated for presence; the split-K partial sums live in the
  * library's own per-device workspace (see lorax_init).
  */

@@ -11,6 +11,7 @@
 // workgroup streams the adapter's rows once for up to kGroup tokens, with 16-byte
 // loads, fp32 accumulation in registers and one wave reduction per output.
 #include "kernels.h"
+#include "sgmv_tiles.h"
 
 namespace lorax {
 
@@ -184,6 +185,68 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_shrink_kernel(
       bgmv_shrink_body<D, RS, 4>(Y, X, A, toks, h_in, row0, P.y_offset, P.y_stride, scale, acc_y, red);
       break;
   }
+}
+
+// ---------------------------------------------------------------------------------
+// SGMV shrink for a handful of rows: the same streaming body, with the token chunks cut from the
+// segments (4 consecutive rows of one segment) instead of gathered by adapter.  A prefill batch of a
+// few dozen tokens has too few 16-row MFMA tiles to occupy the chip and K would have to be split
+// across workgroups; here every (chunk, RS rows of A) pair is a workgroup of its own and the whole
+// workgroup splits K.
+// ---------------------------------------------------------------------------------
+template <typename D, int RS>
+__global__ __launch_bounds__(kBgmvThreads) void sgmv_shrink_rows_kernel(
+    typename D::E* __restrict__ V, const typename D::E* __restrict__ X, const int64_t* __restrict__ W,
+    const int32_t* __restrict__ s_start, const int32_t* __restrict__ s_end, int num_segments, int num_tokens,
+    int h_in, int r, int64_t layer_idx, float scale) {
+  __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<RS * kGroup>::value];
+  using E = typename D::E;
+  const int subs = r / RS;
+  const int v = static_cast<int>(xcd_virtual_id());
+  const int chunk = v / subs;
+  const int row0 = (v % subs) * RS;
+  RowTile rt;
+  if (!find_row_tile(s_start, s_end, num_segments, num_tokens, kGroup, chunk, rt)) return;
+  const int n = rt.row_end - rt.row0;
+  int toks[kGroup];
+#pragma unroll
+  for (int g = 0; g < kGroup; ++g) toks[g] = rt.row0 + min(g, n - 1);
+  const E* A = reinterpret_cast<const E*>(W[rt.seg]) + (layer_idx * r + row0) * static_cast<int64_t>(h_in);
+  switch (n) {
+    case 1:
+      bgmv_shrink_body<D, RS, 1>(V, X, A, toks, h_in, row0, 0, r, scale, true, red);
+      break;
+    case 2:
+      bgmv_shrink_body<D, RS, 2>(V, X, A, toks, h_in, row0, 0, r, scale, true, red);
+      break;
+    case 3:
+      bgmv_shrink_body<D, RS, 3>(V, X, A, toks, h_in, row0, 0, r, scale, true, red);
+      break;
+    default:
+      bgmv_shrink_body<D, RS, 4>(V, X, A, toks, h_in, row0, 0, r, scale, true, red);
+      break;
+  }
+}
+
+template <typename D>
+static hipError_t launch_shrink_rows_dtype(const SgmvArgs& a, hipStream_t stream) {
+  const int64_t chunks = (a.num_tokens + kGroup - 1) / kGroup + a.num_segments;  // upper bound
+  const int rs = chunks * (a.d_out / 8) >= 512 ? 8 : (chunks * (a.d_out / 4) >= 512 ? 4 : 2);
+  const dim3 grid(static_cast<unsigned>(chunks * (a.d_out / rs)));
+  auto args = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(kBgmvThreads), 0, stream, static_cast<typename D::E*>(a.y),
+                       static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end, a.num_segments,
+                       static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, a.scale);
+  };
+  if (rs == 8) args(sgmv_shrink_rows_kernel<D, 8>);
+  else if (rs == 4) args(sgmv_shrink_rows_kernel<D, 4>);
+  else args(sgmv_shrink_rows_kernel<D, 2>);
+  return hipGetLastError();
+}
+
+// v[s:e] += T(scale * x[s:e] @ A_i^T) for [L, r, h_in] stacks, r a multiple of 8; meant for short batches.
+hipError_t launch_sgmv_shrink_rows(const SgmvArgs& a, hipStream_t stream) {
+  return a.dtype == LORAX_F16 ? launch_shrink_rows_dtype<F16>(a, stream) : launch_shrink_rows_dtype<BF16>(a, stream);
 }
 
 // ---------------------------------------------------------------------------------

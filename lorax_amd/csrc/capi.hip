@@ -95,7 +95,7 @@ int check_common(const void* y, const void* x, const void* w_ptrs, int dtype) {
 const Tuning& tuning() {
   static const Tuning t = {env_int("LORAX_BGMV_LORA_BLOCKS"), env_int("LORAX_BGMV_SHRINK_ROWS"), env_int("LORAX_SHRINK_KSPLIT"),
                            env_int("LORAX_SHRINK_MB"), env_int("LORAX_SHRINK_WAVES"), env_int("LORAX_EXPAND_ROWS"),
-                           env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB"), env_int("LORAX_BGMV_EXPAND_COLS"), env_int("LORAX_EXPAND_PANELS"), env_int("LORAX_BGMV_NO_RUNS")};
+                           env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB"), env_int("LORAX_BGMV_EXPAND_COLS"), env_int("LORAX_EXPAND_PANELS"), env_int("LORAX_BGMV_NO_RUNS"), env_int("LORAX_SHRINK_ROWS_MAX")};
   return t;
 }
 
@@ -220,9 +220,9 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
     return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p tmp=%p)", s_start, s_end, tmp);
   if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
   // [L, r, h_in]: multiples of 16 as in the reference (sgmv_config.h:10-15), and any multiple of 8 where the
-  // LDS-staged kernel applies (h_in a multiple of 128)
+  // LDS-staged kernel (h_in a multiple of 128) or the streaming kernel (up to 512 rows) applies
   const bool r_ok = r >= 8 && r <= kMaxRank && r % 8 == 0 &&
-                    (a_layout == LORAX_A_HR || r % 16 == 0 || h_in % 128 == 0);
+                    (a_layout == LORAX_A_HR || r % 16 == 0 || h_in % 128 == 0 || num_tokens <= 512);
   if (!r_ok || h_in <= 0 || h_in % 8 != 0 || num_tokens > INT32_MAX / 2)
     return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in,
                 r, a_layout);

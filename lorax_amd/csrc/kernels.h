@@ -100,6 +100,7 @@ struct Tuning {
   int bgmv_expand_cols;  // LORAX_BGMV_EXPAND_COLS: columns per lane group of the BGMV expand (4, 8, 16)
   int expand_panels;  // LORAX_EXPAND_PANELS: column panels per wave of the transposed-B expand
   int bgmv_no_runs;   // LORAX_BGMV_NO_RUNS: number workgroups problem by problem
+  int shrink_rows_max;  // LORAX_SHRINK_ROWS_MAX: largest token count served by the streaming SGMV shrink (-1 = never)
 };
 const Tuning& tuning();
 
@@ -111,6 +112,8 @@ hipError_t launch_sgmv_expand_t(const SgmvArgs& a, hipStream_t stream);  // B st
 // LDS-staged shrink (sgmv_shrink_lds.hip): [L, r, h_in] layout, h_in a multiple of 128.
 bool sgmv_shrink_lds_applies(const SgmvArgs& a);
 hipError_t launch_sgmv_shrink_lds(const SgmvArgs& a, hipStream_t stream);
+// Streaming shrink for a handful of rows (bgmv.hip): [L, r, h_in] layout, any h_in the BGMV kernels take.
+hipError_t launch_sgmv_shrink_rows(const SgmvArgs& a, hipStream_t stream);
 
 // Workspace layout constants shared by capi.hip and sgmv_shrink.hip.
 constexpr size_t kPartialBytes = 96u << 20;  // fp32 split-K partial sums

@@ -112,7 +112,7 @@ class LoraLinear(nn.Module):
                 # Prefill reads the resident stacks ([L, r, h_in] and [L, h_out, r], the ones decode uses);
                 # the reference's prefill layouts are only touched for shapes the resident-layout shrink
                 # does not take.
-                if rs.lora_a_t_ptr is not None and resident_shrink_applies(r, input.size(1)):
+                if rs.lora_a_t_ptr is not None and resident_shrink_applies(r, input.size(1), input.size(0)):
                     v = lora_a_sgmv_resident(
                         input, get_tmp_tensor(input.device), rs.lora_a_t_ptr, rs.segment_starts, rs.segment_ends,
                         self.layer_id, r,

@@ -149,10 +149,11 @@ def lora_a_sgmv_resident(
     return v
 
 
-def resident_shrink_applies(lora_rank: int, h_in: int) -> bool:
+def resident_shrink_applies(lora_rank: int, h_in: int, num_tokens: int = 1 << 30) -> bool:
     """Ranks the [L, r, h_in] shrink entry accepts: multiples of 16 always, other multiples of 8 when h_in is
-    a multiple of 128."""
-    return 8 <= lora_rank <= MAX_RANK_CUSTOM and lora_rank % 8 == 0 and (lora_rank % 16 == 0 or h_in % 128 == 0)
+    a multiple of 128 or the batch has at most 512 rows."""
+    return 8 <= lora_rank <= MAX_RANK_CUSTOM and lora_rank % 8 == 0 and (
+        lora_rank % 16 == 0 or h_in % 128 == 0 or num_tokens <= 512)
 
 
 def lora_b_sgmv_cutlass(

@@ -68,7 +68,7 @@ def test_sgmv_shrink_validation():
     assert f(P, P, P, P, P, 0, 16, 4096, 16, 0, 0, 1.0, P, big, 0, None) == OK  # no segments
     assert f(P, P, P, P, P, 2, 16, 4096, 16, 7, 0, 1.0, P, big, 0, None) == EINVAL  # layout
     for r, h_in in ((8, 4104), (24, 4104), (144, 4096), (12, 4096)):
-        assert f(P, P, P, P, P, 2, 16, h_in, r, 0, 0, 1.0, P, big, 0, None) == ENOKERNEL, r
+        assert f(P, P, P, P, P, 2, 1000, h_in, r, 0, 0, 1.0, P, big, 0, None) == ENOKERNEL, r
     assert f(P, P, P, P, P, 2, 16, 4100, 16, 0, 0, 1.0, P, big, 0, None) == ENOKERNEL
     assert f(P, P, P, None, P, 2, 16, 4096, 16, 0, 0, 1.0, P, big, 0, None) == EINVAL
     assert f(P, P, P, P, P, 2, 16, 4096, 16, 0, 0, 1.0, P, big, 5, None) == ENOKERNEL  # dtype

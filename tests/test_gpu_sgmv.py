@@ -134,9 +134,10 @@ def test_sgmv_shrink_expand_vs_oracle(dtype, r, h_in, h_out, lens):
     (32, 512, [500] * 8 + [5]),               # 32-row tiles
     (48, 256, [600, 700, 800, 900, 1000]),    # 32-row tiles, odd number of rank blocks
     (128, 256, [40] * 100 + [1] * 60),        # 32-row tiles, rank 128, many short segments
-    (16, 128, [1] * 200),                     # 16-row tiles, one row each
+    (16, 128, [1] * 600),                     # 16-row tiles, one row each
     (64, 192, [3000, 2000, 3000]),            # h_in not a multiple of 128: register-operand kernel
-    (16, 4160, [100, 28]),                    # the same with K split across workgroups
+    (16, 4160, [330, 290]),                   # the same with K split across workgroups
+    (24, 1000, [100, 28, 1]),                 # a few rows: streaming kernel, any rank and h_in multiple of 8
 ])
 def test_sgmv_shrink_tile_variants(r, h_in, lens):
     print(f"case r={r} h_in={h_in} segments={len(lens)} rows={sum(lens)}", flush=True)
@@ -238,7 +239,7 @@ def test_sgmv_shrink_resident_layout_any_rank(dtype, r, h_in, lens):
     for s, e in zip(starts, ends):
         covered[s:e] = True
     assert torch.count_nonzero(v.cpu()[~covered]) == 0
-    if r % 16 != 0:
+    if r % 16 != 0 and T > 512:
         with pytest.raises(RuntimeError, match="No suitable kernel"):
             _native.sgmv_shrink(torch.zeros((T, r), dtype=dtype, device=DEV), x[:, :h_in - 64].contiguous(),
                                 ptr_table(wa_t, DEV), torch.tensor(starts, dtype=torch.int32, device=DEV),
