@@ -228,6 +228,15 @@ def build_bgmv_plan(token_slots: List[int], a_addrs: List[int], b_addrs: List[in
     return records
 
 
+def _segment_order(segs: List[int], seg_adapters: List[int], bounds: List[int]):
+    """Sort key of a rank group's segments: rows of the segment's adapter inside the group, descending, then the
+    adapter index."""
+    rows: Dict[int, int] = defaultdict(int)
+    for s in segs:
+        rows[seg_adapters[s]] += bounds[s + 1] - bounds[s]
+    return lambda s: (-rows[seg_adapters[s]], seg_adapters[s])
+
+
 class _LayoutView(Mapping):
     """adapter index -> one layout of its stack (an attribute of LoraWeights), fetched on access."""
 
@@ -337,6 +346,11 @@ class BatchLoraWeights(BatchAdapterWeights):
         token_adapters = None if use_sgmv else meta.adapter_indices.tolist()
         rank_data: Dict[int, RankSegments] = {}
         for rank, segs in by_rank.items():
+            if use_sgmv:
+                # the order of a group's segments is free: keep the segments of one adapter together, so that
+                # their tiles run back to back and share the adapter's weights in L2, adapters with the most
+                # rows first (the long tiles of a launch start early)
+                segs.sort(key=_segment_order(segs, seg_adapters, meta.adapter_segments.tolist()))
             tmp_shrink = tmp_expand = starts = ends = token_slots = plan = None
             if use_sgmv:
                 tmp_shrink, tmp_expand = get_tmp_tensors(len(segs), rank, device)
@@ -590,6 +604,7 @@ def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAda
             if use_sgmv:
                 tmp_shrink, tmp_expand = get_tmp_tensors(n, g.rank, device)
                 segs = [s for s, a in enumerate(seg_adapters) if a in loras and loras[a].lora_a_r == g.rank]
+                segs.sort(key=_segment_order(segs, seg_adapters, bounds.tolist()))
                 rank_data[g.rank] = RankSegments(
                     rank=g.rank,
                     lora_a_ptr=(lambda segs=segs, table=table: table("weights_a")[segs]),

@@ -107,8 +107,26 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
     }
 
     for (size_t g = 0; g < group_of_rank.size(); ++g) {
-      const std::vector<int32_t>& segs = group_segs[g];
+      std::vector<int32_t>& segs = group_segs[g];
       const int32_t n = static_cast<int32_t>(segs.size());
+      // Segment tables: the order of a group's segments is free.  The segments of one adapter are put next to
+      // each other: their tiles then run back to back on one XCD and the second one finds the adapter's
+      // weights in L2 - decode tokens inside a prefill batch are one-row segments, and an adapter that serves
+      // several of them would otherwise be streamed once per token.  Adapters with the most rows come first,
+      // so that the long tiles of a launch start early.  Stable: (rows of the adapter, descending; adapter).
+      if (use_sgmv) {
+        std::vector<int64_t> rows_of(num_segments, 0);
+        for (int32_t x : segs) {
+          int64_t rows = 0;
+          for (int32_t y : segs)
+            if (segment_owners[y] == segment_owners[x]) rows += segment_bounds[y + 1] - segment_bounds[y];
+          rows_of[x] = rows;
+        }
+        std::stable_sort(segs.begin(), segs.end(), [&](int32_t x, int32_t y) {
+          if (rows_of[x] != rows_of[y]) return rows_of[x] > rows_of[y];
+          return segment_owners[x] < segment_owners[y];
+        });
+      }
       lorax_table_group_t desc{};
       desc.layer_type = lt;
       desc.rank = group_of_rank[g];

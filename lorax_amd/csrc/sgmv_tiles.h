@@ -18,43 +18,75 @@ struct RowTile {
   int row_end;  // one past the last row of the tile (<= end of segment)
 };
 
+// One chunk of 64 segments: lane `lane` holds the clamped bounds (s, e) of segment seg0 + lane.  If `tile`
+// (counted from the first tile of the chunk, `rel`) falls into the chunk, fills `out` and returns true;
+// otherwise adds the chunk's tiles to `base`.
+__device__ __forceinline__ bool tile_in_chunk(int s, int e, int seg0, int rows_per_tile, int tile, int& base,
+                                              RowTile& out) {
+  const int lane = lane_id();
+  const int len = max(e - s, 0);
+  const int nt = (len + rows_per_tile - 1) / rows_per_tile;
+  int inc = nt;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int t = __shfl_up(inc, d, kWave);
+    if (lane >= d) inc += t;
+  }
+  const int chunk_total = __shfl(inc, kWave - 1, kWave);
+  const int rel = tile - base;
+  if (rel < chunk_total) {
+    const bool hit = (rel >= inc - nt) && (rel < inc);
+    const uint64_t mask = __ballot(hit);
+    const int src = __ffsll(static_cast<unsigned long long>(mask)) - 1;
+    const int ti = rel - __shfl(inc - nt, src, kWave);
+    const int s_f = __shfl(s, src, kWave);
+    const int e_f = __shfl(e, src, kWave);
+    out.seg = seg0 + src;
+    out.row0 = s_f + ti * rows_per_tile;
+    out.row_end = min(e_f, out.row0 + rows_per_tile);
+    return true;
+  }
+  base += chunk_total;
+  return false;
+}
+
 // Wave-uniform.  Returns false when `tile` is past the last tile of the launch.
+// The bounds of the first kTilePreload * 64 segments are all requested before the first one is looked at,
+// so that a batch of a few hundred segments (decode tokens inside a prefill batch) costs one memory round
+// trip instead of one per 64 segments.
+constexpr int kTilePreload = 4;
+
 __device__ __forceinline__ bool find_row_tile(const int32_t* __restrict__ s_start,
                                               const int32_t* __restrict__ s_end,
                                               int num_segments, int num_tokens,
                                               int rows_per_tile, int tile, RowTile& out) {
+  if (num_segments <= 0) return false;
   const int lane = lane_id();
+  int s_pre[kTilePreload], e_pre[kTilePreload];
+#pragma unroll
+  for (int c = 0; c < kTilePreload; ++c) {
+    // unconditional loads of clamped indices: every load is in flight before the first wait
+    const int seg = min(c * kWave + lane, num_segments - 1);
+    s_pre[c] = s_start[seg];
+    e_pre[c] = s_end[seg];
+  }
   int base = 0;
-  for (int seg0 = 0; seg0 < num_segments; seg0 += kWave) {
+#pragma unroll
+  for (int c = 0; c < kTilePreload; ++c) {
+    if (c * kWave >= num_segments) return false;
+    const bool live = c * kWave + lane < num_segments;
+    const int s = live ? max(s_pre[c], 0) : 0;
+    const int e = live ? min(e_pre[c], num_tokens) : 0;
+    if (tile_in_chunk(s, e, c * kWave, rows_per_tile, tile, base, out)) return true;
+  }
+  for (int seg0 = kTilePreload * kWave; seg0 < num_segments; seg0 += kWave) {
     const int seg = seg0 + lane;
     int s = 0, e = 0;
     if (seg < num_segments) {
       s = max(s_start[seg], 0);
       e = min(s_end[seg], num_tokens);
     }
-    const int len = max(e - s, 0);
-    const int nt = (len + rows_per_tile - 1) / rows_per_tile;
-    int inc = nt;
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const int t = __shfl_up(inc, d, kWave);
-      if (lane >= d) inc += t;
-    }
-    const int chunk_total = __shfl(inc, kWave - 1, kWave);
-    const int rel = tile - base;
-    if (rel < chunk_total) {
-      const bool hit = (rel >= inc - nt) && (rel < inc);
-      const uint64_t mask = __ballot(hit);
-      const int src = __ffsll(static_cast<unsigned long long>(mask)) - 1;
-      const int ti = rel - __shfl(inc - nt, src, kWave);
-      const int s_f = __shfl(s, src, kWave);
-      const int e_f = __shfl(e, src, kWave);
-      out.seg = seg0 + src;
-      out.row0 = s_f + ti * rows_per_tile;
-      out.row_end = min(e_f, out.row0 + rows_per_tile);
-      return true;
-    }
-    base += chunk_total;
+    if (tile_in_chunk(s, e, seg0, rows_per_tile, tile, base, out)) return true;
   }
   return false;
 }
