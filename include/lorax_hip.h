@@ -106,6 +106,8 @@ int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* ind
  *   [6] device address of the adapter's B^T stack [L, h_out, r] (read by expand launches)
  *   [7] reserved
  * where every chunk holds tokens of ONE adapter and every routed token is in exactly one chunk.
+ * A record whose word [0] is 0 is padding and is skipped, so a plan can be kept at a fixed number of
+ * records for graph replay (the reference pads its tables the same way, utils/graph.py:71-73,421-425).
  * With a plan, w_ptrs and indices are not read and may be NULL.
  */
 typedef struct lorax_bgmv_problem {

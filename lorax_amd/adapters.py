@@ -228,6 +228,17 @@ def build_bgmv_plan(token_slots: List[int], a_addrs: List[int], b_addrs: List[in
     return records
 
 
+def pad_bgmv_plan(plan: torch.Tensor, num_records: int) -> torch.Tensor:
+    """`plan` extended with all-zero records to a fixed number of records: the kernels skip them, so a decode
+    step captured in a graph can be replayed with the plans of later batches copied into the same tensor
+    (the reference pads pointer tables with 0 and indices with -1 for the same purpose, utils/graph.py:71-73)."""
+    if plan.size(0) > num_records:
+        raise ValueError(f"plan has {plan.size(0)} records, more than the fixed size {num_records}")
+    padded = torch.zeros((num_records, BGMV_PLAN_WORDS), dtype=plan.dtype, device=plan.device)
+    padded[: plan.size(0)] = plan
+    return padded
+
+
 def _segment_order(segs: List[int], seg_adapters: List[int], bounds: List[int]):
     """Sort key of a rank group's segments: rows of the segment's adapter inside the group, descending, then the
     adapter index."""

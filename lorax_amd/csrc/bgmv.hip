@@ -585,6 +585,7 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch
   const int col_end = min(col0 + cols_per_wg, h_out);
   const int64_t* rec = P.plan + static_cast<int64_t>(vb.y) * kPlanRecordWords;
   const int n = static_cast<int>(rec[0]);
+  if (n <= 0) return;  // an all-zero record: padding of a plan kept at a fixed size for graph replay
   int toks[kGroup];
 #pragma unroll
   for (int g = 0; g < kGroup; ++g) toks[g] = static_cast<int>(rec[1 + g]);

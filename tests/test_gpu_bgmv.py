@@ -324,3 +324,66 @@ def test_bgmv_single_launch_shrink_expand(dtype, r, h_in, sizes):
     assert_close(y, y_ref, "single-launch LoRA")
     with pytest.raises(RuntimeError, match="No suitable kernel"):
         _native.bgmv_lora_multi(problems, 32, 1)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_padded_plan_and_graph_replay_with_a_new_batch(fused):
+    """A plan padded with all-zero records gives the same result as the plan itself, and a captured decode step
+    can be replayed for a different batch by copying that batch's padded plan, inputs and y into place."""
+    from lorax_amd import _native
+    from lorax_amd.adapters import build_bgmv_plan, pad_bgmv_plan
+
+    dtype, T, h_in, h_out, r, n = torch.bfloat16, 48, 1024, 1024, 8, 6
+    gen = torch.Generator().manual_seed(31)
+    wa_t = _stacks(n, 2, r, h_in, gen, dtype)
+    wb_t = _stacks(n, 2, h_out, r, gen, dtype)
+    a_ptr, b_ptr = ptr_table(wa_t, DEV), ptr_table(wb_t, DEV)
+    max_records = T  # one token per chunk at worst
+
+    def batch(seed):
+        g = torch.Generator().manual_seed(seed)
+        idx = _indices(T, n, g, drop=0.2)
+        records = build_bgmv_plan(idx.tolist(), a_ptr.tolist(), b_ptr.tolist())
+        plan = torch.tensor(records, dtype=torch.int64, device=DEV).reshape(-1, 8)
+        x = randn((T, h_in), 1.0, g, dtype, DEV)
+        y0 = randn((T, h_out), 0.5, g, dtype, DEV)
+        v_ref = torch.zeros((T, r), dtype=dtype)
+        O.bgmv_ref(v_ref, x.cpu(), [w.cpu() for w in wa_t], idx.tolist(), 1)
+        y_ref = y0.cpu().clone()
+        O.bgmv_ref(y_ref, v_ref, [w.cpu() for w in wb_t], idx.tolist(), 1)
+        return idx.to(DEV), plan, x, y0, y_ref
+
+    idx1, plan1, x1, y01, ref1 = batch(1)
+    idx2, plan2, x2, y02, ref2 = batch(2)
+    assert plan1.size(0) != plan2.size(0) or not torch.equal(plan1, plan2)
+
+    x, y = x1.clone(), y01.clone()
+    plan = pad_bgmv_plan(plan1, max_records)
+    v = torch.empty((T, r), dtype=dtype, device=DEV)
+    idx = idx1.clone()
+
+    def step():
+        if fused:
+            _native.bgmv_lora_multi([(y, x, plan, 0, None)], r, 1)
+        else:
+            _native.bgmv_multi([(v, x, a_ptr, idx, 0, None)], 1, 1.0, accumulate=False, plans=[plan])
+            _native.bgmv_multi([(y, v, b_ptr, idx, 0, None)], 1, 1.0, accumulate=True, plans=[plan])
+
+    step()
+    torch.cuda.synchronize()
+    assert_close(y, ref1, "padded plan, eager")
+    unpadded = y01.clone()
+    if fused:
+        _native.bgmv_lora_multi([(unpadded, x1, plan1, 0, None)], r, 1)
+        assert torch.equal(unpadded, y)
+
+    y.copy_(y01)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for x_new, y_new, plan_new, idx_new, ref in ((x2, y02, plan2, idx2, ref2), (x1, y01, plan1, idx1, ref1)):
+        x.copy_(x_new), y.copy_(y_new), idx.copy_(idx_new)
+        plan.copy_(pad_bgmv_plan(plan_new, max_records))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_close(y, ref, "graph replay with another batch's plan")
