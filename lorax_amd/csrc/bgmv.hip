@@ -571,6 +571,32 @@ __device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
 }
 
 template <typename D, int R, int U, int NBLK, bool VEC4>
+__device__ __forceinline__ void bgmv_lora_tokens(int n, typename D::E* Y, const typename D::E* X,
+                                                 const typename D::E* A, const typename D::E* B,
+                                                 const int (&toks)[kGroup], int h_in, int h_out, int col0, int col_end,
+                                                 int64_t y_offset, int64_t y_stride, float scale, float* red,
+                                                 typename D::E* vsh) {
+  switch (n) {
+    case 1:
+      bgmv_lora_body<D, R, U, NBLK, 1, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, y_offset, y_stride, scale, red,
+                                             vsh);
+      break;
+    case 2:
+      bgmv_lora_body<D, R, U, NBLK, 2, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, y_offset, y_stride, scale, red,
+                                             vsh);
+      break;
+    case 3:
+      bgmv_lora_body<D, R, U, NBLK, 3, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, y_offset, y_stride, scale, red,
+                                             vsh);
+      break;
+    default:
+      bgmv_lora_body<D, R, U, NBLK, 4, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, y_offset, y_stride, scale, red,
+                                             vsh);
+      break;
+  }
+}
+
+template <typename D, int R, int U, int NBLK, bool VEC4>
 __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch batch, int h_in,
                                                                  int64_t layer_idx, float scale) {
   using E = typename D::E;
@@ -593,24 +619,15 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch
   const E* B = reinterpret_cast<const E*>(rec[6]) + layer_idx * h_out * static_cast<int64_t>(R);
   E* Y = static_cast<E*>(P.y);
   const E* X = static_cast<const E*>(P.x);
-  switch (n) {
-    case 1:
-      bgmv_lora_body<D, R, U, NBLK, 1, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
-                                 red, vsh);
-      break;
-    case 2:
-      bgmv_lora_body<D, R, U, NBLK, 2, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
-                                 red, vsh);
-      break;
-    case 3:
-      bgmv_lora_body<D, R, U, NBLK, 3, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
-                                 red, vsh);
-      break;
-    default:
-      bgmv_lora_body<D, R, U, NBLK, 4, VEC4>(Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
-                                 red, vsh);
-      break;
-  }
+  // A narrow projection batched with wide ones (k and v next to q) fills one expand block only: it runs the
+  // one-block body, which neither loads nor multiplies the three empty blocks.
+  constexpr int kBlockCols = (kBgmvThreads / (R / 8)) * U;
+  if (NBLK > 1 && col_end - col0 <= kBlockCols)
+    bgmv_lora_tokens<D, R, U, 1, VEC4>(n, Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride, scale,
+                                       red, vsh);
+  else
+    bgmv_lora_tokens<D, R, U, NBLK, VEC4>(n, Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride,
+                                          scale, red, vsh);
 }
 
 // ---------------------------------------------------------------------------------
