@@ -10,6 +10,8 @@
 // Here the tokens of one adapter are grouped inside the kernel (group_tokens) and a
 // workgroup streams the adapter's rows once for up to kGroup tokens, with 16-byte
 // loads, fp32 accumulation in registers and one wave reduction per output.
+#include <utility>
+
 #include "kernels.h"
 #include "sgmv_tiles.h"
 
@@ -596,13 +598,59 @@ __device__ __forceinline__ void bgmv_lora_tokens(int n, typename D::E* Y, const 
   }
 }
 
+// Workgroup placement for a batch of one wide and several narrow projections (q with k and v) when the
+// launch has between one and two workgroups per CU.  The hardware hands workgroup h to XCD h % 8, and
+// inside an XCD the workgroup in slot s = h / 8 shares its CU with the one in slot s + 32 (measured: 32
+// CUs per XCD are filled once before any gets a second workgroup).  Two workgroups on a CU halve each
+// other's vector-ALU rate, and the launch ends with its slowest CU, so the wide projection's workgroups
+// are put into the slots that stay alone on their CU and the narrow ones into the shared slots.
+// XCD k owns the token chunks [k * chunks_per_xcd, ...); problem 0 is the wide one.  Returns false for
+// a slot without work.
+__device__ __forceinline__ bool balanced_slot(int count, int chunks, int chunks_per_xcd, VirtualBlock& vb) {
+  constexpr int kCusPerXcd = 32;
+  const int xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+  const int slots = chunks_per_xcd * count;       // per XCD, between 33 and 64
+  const int first = xcd * chunks_per_xcd;
+  const int heavy = max(min(chunks - first, chunks_per_xcd), 0);  // wide-projection workgroups of this XCD
+  const int light = heavy * (count - 1);
+  const int shared = slots - kCusPerXcd;          // slots [0, shared) pair with [32, 32 + shared)
+  const int alone = kCusPerXcd - shared;          // slots [shared, 32)
+  const int heavy_alone = min(heavy, alone);
+  int h = -1, l = -1;                             // index among the XCD's heavy / light workgroups
+  if (slot >= shared && slot < kCusPerXcd) {
+    const int u = slot - shared;
+    if (u < heavy_alone) h = u; else l = u - heavy_alone;
+  } else {
+    const int i = slot < shared ? slot : shared + (slot - kCusPerXcd);
+    const int heavy_shared = heavy - heavy_alone;
+    if (i < heavy_shared) h = heavy_alone + i; else l = (alone - heavy_alone) + (i - heavy_shared);
+  }
+  vb.x = 0;
+  if (h >= 0) {
+    if (h >= heavy) return false;
+    vb.y = first + h;
+    vb.z = 0;
+    return true;
+  }
+  if (l >= light) return false;
+  vb.y = first + l / (count - 1);
+  vb.z = 1 + l % (count - 1);
+  return true;
+}
+
 template <typename D, int R, int U, int NBLK, bool VEC4>
 __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch batch, int h_in,
-                                                                 int64_t layer_idx, float scale) {
+                                                                 int64_t layer_idx, float scale, int count,
+                                                                 int balanced_chunks, int chunks_per_xcd) {
   using E = typename D::E;
   __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<R * kGroup>::value];
   __shared__ __attribute__((aligned(16))) E vsh[R * kGroup];
-  const VirtualBlock vb = xcd_virtual_block();
+  VirtualBlock vb;
+  if (balanced_chunks > 0) {
+    if (!balanced_slot(count, balanced_chunks, chunks_per_xcd, vb)) return;
+  } else {
+    vb = xcd_virtual_block();
+  }
   const BgmvProblem& P = batch.p[vb.z];
   const int h_out = P.width;
   constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
@@ -722,20 +770,39 @@ template <typename D, int R, int NBLK>
 static hipError_t launch_lora_blk(const BgmvArgs& a, hipStream_t stream) {
   constexpr int U = 4;
   constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
+  BgmvBatch batch = a.batch;
   dim3 grid((a.wide_max + cols_per_wg - 1) / cols_per_wg, static_cast<unsigned>(a.grid_rows), a.count);
+  // One wide projection batched with narrow ones, one column slice each, one to two workgroups per CU:
+  // place the wide projection's workgroups on CUs of their own (balanced_slot).
+  int balanced_chunks = 0, chunks_per_xcd = 0;
+  if (grid.x == 1 && a.count > 1 && !tuning().bgmv_no_balance) {
+    int widest = 0;
+    for (int i = 1; i < a.count; ++i)
+      if (batch.p[i].width > batch.p[widest].width) widest = i;
+    bool same_chunks = true;
+    for (int i = 0; i < a.count; ++i) same_chunks = same_chunks && batch.p[i].num_groups == batch.p[0].num_groups;
+    const int per_xcd = (static_cast<int>(a.grid_rows) + kXcds - 1) / kXcds;
+    const int slots = per_xcd * a.count;
+    if (same_chunks && slots > 32 && slots <= 64) {
+      std::swap(batch.p[0], batch.p[widest]);  // problems are independent: their order is free
+      balanced_chunks = static_cast<int>(a.grid_rows);
+      chunks_per_xcd = per_xcd;
+      grid = dim3(kXcds * slots);
+    }
+  }
   // 8-byte y accesses need every problem's rows 8-byte aligned and no ragged last column group
   bool vec4 = true;
   for (int i = 0; i < a.count; ++i) {
-    const BgmvProblem& p = a.batch.p[i];
+    const BgmvProblem& p = batch.p[i];
     vec4 = vec4 && p.width % 4 == 0 && p.y_stride % 4 == 0 && p.y_offset % 4 == 0 &&
            reinterpret_cast<uintptr_t>(p.y) % 8 == 0;
   }
   if (vec4)
-    hipLaunchKernelGGL((bgmv_lora_kernel<D, R, U, NBLK, true>), grid, dim3(kBgmvThreads), 0, stream, a.batch, a.h_in,
-                       a.layer_idx, a.scale);
+    hipLaunchKernelGGL((bgmv_lora_kernel<D, R, U, NBLK, true>), grid, dim3(kBgmvThreads), 0, stream, batch, a.h_in,
+                       a.layer_idx, a.scale, a.count, balanced_chunks, chunks_per_xcd);
   else
-    hipLaunchKernelGGL((bgmv_lora_kernel<D, R, U, NBLK, false>), grid, dim3(kBgmvThreads), 0, stream, a.batch,
-                       a.h_in, a.layer_idx, a.scale);
+    hipLaunchKernelGGL((bgmv_lora_kernel<D, R, U, NBLK, false>), grid, dim3(kBgmvThreads), 0, stream, batch,
+                       a.h_in, a.layer_idx, a.scale, a.count, balanced_chunks, chunks_per_xcd);
   return hipGetLastError();
 }
 

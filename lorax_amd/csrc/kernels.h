@@ -100,6 +100,7 @@ struct Tuning {
   int bgmv_expand_cols;  // LORAX_BGMV_EXPAND_COLS: columns per lane group of the BGMV expand (4, 8, 16)
   int expand_panels;  // LORAX_EXPAND_PANELS: column panels per wave of the transposed-B expand
   int bgmv_no_runs;   // LORAX_BGMV_NO_RUNS: number workgroups problem by problem
+  int bgmv_no_balance;  // LORAX_BGMV_NO_BALANCE: plain workgroup numbering in the single-launch BGMV
   int shrink_rows_max;  // LORAX_SHRINK_ROWS_MAX: largest token count served by the streaming SGMV shrink (-1 = never)
 };
 const Tuning& tuning();
