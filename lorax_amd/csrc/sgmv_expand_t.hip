@@ -1,20 +1,24 @@
 // SGMV expand over the transposed B stack: y[s:e, off:off+h_out] += T(v[s:e, :r] @ B_i), with B_i
 // stored as B_i^T = [h_out, r] (the layout the decode path keeps resident anyway).
 //
-// Same arithmetic and rounding as sgmv_expand.hip (the transposed MFMA product: B^T as the first
-// operand, v as the second, so that a lane ends up with 8 adjacent columns of one y row and y moves
-// in 16-byte pieces), but with B^T in memory the first operand needs no transposition: lane (c, g)
-// of accumulator j reads the 16 bytes B^T[column(j, c)][32 s + 8 g ...] straight from global memory,
-// and the 64-column panel of a wave is one contiguous run of 64 * r * 2 bytes.  That removes the LDS
-// staging, its two barriers and the 2-byte LDS gathers from every tile's prologue - which, for the
-// short segments a prefill batch is full of, took longer than the rows themselves - and it makes
-// the weight reads of single-row segments (decode tokens inside a prefill batch) sequential.
+// Same arithmetic and rounding as sgmv_expand.hip.  The MFMA product is v (16 rows of a block, first
+// operand) times B (second operand), and with B^T in memory the second operand needs no transposition:
+// lane (c, g) of accumulator j reads the 16 bytes B^T[column(j, c)][32 s + 8 g ...] straight from global
+// memory.  There is no LDS staging, no barrier and no LDS gather in a tile's prologue - which, for the
+// short segments a prefill batch is full of, took longer than the rows themselves.
 //
-// Work split: a workgroup owns one row tile and 4 * panels_per_wave column panels of 64; wave w takes
-// panels w, w + 4, ... and walks ALL 16-row blocks of the tile for each (the four waves touch 512
-// adjacent bytes of every row).  The tile search runs once per workgroup.  There is no separate path
-// for segments of a few rows: rows past the tile's end are clamped for loads and predicated for
-// stores, and MFMA work on padding is free in a kernel that waits on memory.
+// The columns of a wave's panel are dealt to the accumulators so that a lane ends up with NJ ADJACENT
+// columns of four rows (see the kernel).  A y access of the wave is then four whole runs of 32 * NJ
+// bytes, one per row, and the texture path handles it as a few cache lines.  (With the product the other
+// way round - B^T first, v second - a lane holds 8 adjacent columns of ONE row and neighbouring lanes
+// hold different rows: every 16-byte piece is then a separate cache-line lookup, 64 per instruction, and
+// the kernel is bound by the address path of the CU at 60 % of what it reaches now; counters:
+// TA_ADDR_STALLED_BY_TC_CYCLES at 60 % and TA_BUSY at 80 % of the kernel's duration.)
+//
+// Work split: a workgroup owns one row tile and 4 * panels_per_wave column panels of 16 * NJ; wave w takes
+// panels w, w + 4, ... and walks ALL 16-row blocks of the tile for each.  The tile search runs once per
+// workgroup.  There is no separate path for segments of a few rows: rows past the tile's end are clamped
+// for loads and predicated for stores, and MFMA work on padding is free in a kernel that waits on memory.
 #include "kernels.h"
 #include "sgmv_tiles.h"
 
@@ -22,16 +26,13 @@ namespace lorax {
 
 constexpr int kExpTWaves = 4;
 constexpr int kExpTThreads = kExpTWaves * kWave;
-constexpr int kExpTCols = 64;   // output columns per wave and panel
-constexpr int kExpTStages = 3;  // register stages of the row-block pipeline
+constexpr int kExpTStages = 2;  // register stages of the row-block pipeline (a third one costs occupancy)
+constexpr int kExpTLaneCols = 4;  // adjacent output columns per lane
 
-// Output column (0..63) that row `a` of the first MFMA operand of accumulator j stands for: lane
-// group g = a / 4 ends up with columns [8g, 8g+8) in accumulators 0,1 and [32+8g, 32+8g+8) in 2,3.
-__device__ __forceinline__ int panel_col_t(int j, int a) {
-  return (j >> 1) * 32 + (a >> 2) * 8 + (j & 1) * 4 + (a & 3);
-}
-
-template <typename D, int KS>
+// NJ accumulators per wave, a panel of 16 * NJ output columns.  Accumulator j stands for the columns
+// n0 + NJ * c + j (c = lane & 15), so a lane ends up with NJ ADJACENT columns of the rows 4g .. 4g + 3
+// (g = lane >> 4) of a 16-row block, and the 16 lanes of one g cover 32 * NJ contiguous bytes of a row.
+template <typename D, int KS, int NJ>
 __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     typename D::E* __restrict__ Y, const typename D::E* __restrict__ V,
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
@@ -40,16 +41,19 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     int tile_slots, int accumulate_into_y) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
+  typedef E yvec __attribute__((ext_vector_type(NJ)));
+  constexpr int kCols = 16 * NJ;
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // wave-uniform, in a scalar register
   const int c = lane & 15;
   const int g = lane >> 4;
-  const int num_panels = (h_out + kExpTCols - 1) / kExpTCols;
+  const int num_panels = (h_out + kCols - 1) / kCols;
   // Workgroup numbering: row tiles fastest, then panel groups, and consecutive numbers on one XCD.  The
   // row tiles of a long segment read the same panels of B^T; as neighbours on one XCD they find them in
   // its L2 instead of fetching them once per tile.
   const int vid = static_cast<int>(xcd_virtual_id());
   const int panel0 = (vid / tile_slots) * kExpTWaves * panels_per_wave;
+  const bool acc_y = accumulate_into_y != 0;
 
   bool k_ok[KS];
   int k_off[KS];
@@ -68,59 +72,62 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     for (int pp = 0; pp < panels_per_wave; ++pp) {
       const int panel = panel0 + pp * kExpTWaves + wave;
       if (panel >= num_panels) break;
-      const int n0 = panel * kExpTCols;
-      const bool col_ok0 = n0 + g * 8 < h_out;
-      const bool col_ok1 = n0 + 32 + g * 8 < h_out;
-      // Loads are unconditional: rows past the tile are clamped to its last row and columns past
-      // h_out to the panel's first vector (both valid memory); only the stores are predicated.
-      const int coff0 = col_ok0 ? g * 8 : 0;
-      const int coff1 = col_ok1 ? 32 + g * 8 : 0;
-      auto load_block = [&](int mb, vec8(&vf)[KS], vec8& y0, vec8& y1) {
-        const int row = min(rt.row0 + mb * 16 + c, rt.row_end - 1);
-        const E* vp = V + static_cast<int64_t>(row) * r;
+      const int n0 = panel * kCols;
+      // h_out is a multiple of 8 and so is NJ * c: a lane's NJ columns are inside the matrix or outside it
+      // as a whole.  Loads are unconditional: rows past the tile are clamped to its last row and a lane
+      // past h_out reads the panel's first columns (both valid memory); only the stores are predicated.
+      const bool col_ok = n0 + NJ * c < h_out;
+      const int col = col_ok ? n0 + NJ * c : n0;
+      // Addresses inside a tile: a wave-uniform 64-bit base and a 32-bit offset per lane (a tile spans at
+      // most rows_per_tile * y_stride elements).
+      const E* vtile = V + static_cast<int64_t>(rt.row0) * r;
+      E* ytile = Y + static_cast<int64_t>(rt.row0) * y_stride + y_offset + n0;
+      const uint32_t ycol = static_cast<uint32_t>(col - n0);
+      const uint32_t ystride = static_cast<uint32_t>(y_stride);
+      const int last = rt.row_end - rt.row0 - 1;
+      auto load_block = [&](int mb, vec8(&vf)[KS], yvec(&yv)[4]) {
+        const uint32_t voff = static_cast<uint32_t>(min(mb * 16 + c, last)) * static_cast<uint32_t>(r);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) vf[s] = load8<D>(vp + k_off[s]);
-        const E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0;
-        y0 = load8<D>(yp + coff0);
-        y1 = load8<D>(yp + coff1);
+        for (int s = 0; s < KS; ++s) vf[s] = load8<D>(vtile + (voff + k_off[s]));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t row = static_cast<uint32_t>(min(mb * 16 + g * 4 + i, last));
+          yv[i] = *(const LORAX_GLOBAL yvec*)(ytile + (row * ystride + ycol));
+        }
       };
       auto block_of = [&](int i) { return min(i, nmb - 1); };
 
       // first row blocks and the panel's operands go out together: one memory round trip
-      vec8 vr[kExpTStages][KS], y0r[kExpTStages], y1r[kExpTStages];
+      vec8 vr[kExpTStages][KS];
+      yvec yr[kExpTStages][4];
 #pragma unroll
-      for (int s = 0; s < kExpTStages - 1; ++s) load_block(block_of(s), vr[s], y0r[s], y1r[s]);
-      vec8 bf[4][KS];
+      for (int s = 0; s < kExpTStages - 1; ++s) load_block(block_of(s), vr[s], yr[s]);
+      vec8 bf[NJ][KS];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int col = min(n0 + panel_col_t(j, c), h_out - 1);
+      for (int j = 0; j < NJ; ++j) {
 #pragma unroll
         for (int s = 0; s < KS; ++s)
-          bf[j][s] = keep_if<D>(k_ok[s], load8<D>(BT + static_cast<int64_t>(col) * r + k_off[s]));
+          bf[j][s] = keep_if<D>(k_ok[s], load8<D>(BT + static_cast<int64_t>(col + j) * r + k_off[s]));
       }
 
-      auto finish_block = [&](bool live, int mb, vec8(&vf)[KS], vec8 y0, vec8 y1) {
-        f32x4 acc[4];
+      auto finish_block = [&](bool live, int mb, vec8(&vf)[KS], yvec(&yv)[4]) {
+        f32x4 acc[NJ];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NJ; ++j) {
           acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int s = 0; s < KS; ++s) acc[j] = D::mfma16(bf[j][s], vf[s], acc[j]);
+          for (int s = 0; s < KS; ++s) acc[j] = D::mfma16(vf[s], bf[j][s], acc[j]);
         }
-        const int row = rt.row0 + mb * 16 + c;
-        const bool ok = live && row < rt.row_end;
-        E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0;
-        y0 = keep_if<D>(accumulate_into_y != 0, y0);  // overwrite mode: the old y counts as zero
-        y1 = keep_if<D>(accumulate_into_y != 0, y1);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          y0[i] = accumulate<D>(y0[i], acc[0][i]);
-          y0[4 + i] = accumulate<D>(y0[4 + i], acc[1][i]);
-          y1[i] = accumulate<D>(y1[i], acc[2][i]);
-          y1[4 + i] = accumulate<D>(y1[4 + i], acc[3][i]);
+          const int row = mb * 16 + g * 4 + i;
+          yvec out;
+#pragma unroll
+          for (int j = 0; j < NJ; ++j)  // overwrite mode: the old y counts as zero
+            out[j] = accumulate<D>(acc_y ? yv[i][j] : static_cast<E>(0.0f), acc[j][i]);
+          if (live && col_ok && row <= last)
+            *(LORAX_GLOBAL yvec*)(ytile + (static_cast<uint32_t>(row) * ystride + ycol)) = out;
         }
-        if (ok && col_ok0) store8<D>(yp + g * 8, y0);
-        if (ok && col_ok1) store8<D>(yp + 32 + g * 8, y1);
       };
 
       // Ring of kExpTStages register stages with static indices: the y and v loads of the next
@@ -130,23 +137,26 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
 #pragma unroll
         for (int s = 0; s < kExpTStages; ++s) {
           constexpr int kAhead = kExpTStages - 1;
-          load_block(block_of(i + s + kAhead), vr[(s + kAhead) % kExpTStages], y0r[(s + kAhead) % kExpTStages],
-                     y1r[(s + kAhead) % kExpTStages]);
+          load_block(block_of(i + s + kAhead), vr[(s + kAhead) % kExpTStages], yr[(s + kAhead) % kExpTStages]);
           __builtin_amdgcn_sched_barrier(0);
-          finish_block(i + s < nmb, block_of(i + s), vr[s], y0r[s], y1r[s]);
+          finish_block(i + s < nmb, block_of(i + s), vr[s], yr[s]);
         }
       }
     }
   }
 }
 
-template <typename D, int KS>
+template <typename D, int KS, int NJ>
 static hipError_t launch_expand_t_ks(const SgmvArgs& a, hipStream_t stream) {
   // 256-row tiles: the prologue is one memory round trip, so taller tiles buy nothing and even out worse
   int rows_per_tile = 256;
   if (tuning().expand_rows > 0) rows_per_tile = (tuning().expand_rows + 15) / 16 * 16;
+  // the kernel addresses a tile with 32-bit element offsets
+  if (a.y_stride * rows_per_tile >= (1ll << 32) || static_cast<int64_t>(a.d_in) * rows_per_tile >= (1ll << 32))
+    return hipErrorInvalidValue;
   const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
-  const int num_panels = (a.d_out + kExpTCols - 1) / kExpTCols;
+  constexpr int kCols = 16 * NJ;
+  const int num_panels = (a.d_out + kCols - 1) / kCols;
   // Panels per wave: more of them amortise the tile search, fewer give more workgroups; keep a few
   // thousand workgroups in the launch.
   int ppw = 4;
@@ -155,7 +165,7 @@ static hipError_t launch_expand_t_ks(const SgmvArgs& a, hipStream_t stream) {
   const int64_t panel_groups = (num_panels + kExpTWaves * ppw - 1) / (kExpTWaves * ppw);
   const int tile_slots = static_cast<int>(tiles < 65535 ? tiles : 65535);
   dim3 grid(static_cast<unsigned>(panel_groups * tile_slots));
-  hipLaunchKernelGGL((sgmv_expand_t_kernel<D, KS>), grid, dim3(kExpTThreads), 0, stream,
+  hipLaunchKernelGGL((sgmv_expand_t_kernel<D, KS, NJ>), grid, dim3(kExpTThreads), 0, stream,
                      static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start,
                      a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.y_offset,
                      a.y_stride, a.layer_idx, rows_per_tile, ppw, tile_slots, a.accumulate);
@@ -166,13 +176,13 @@ template <typename D>
 static hipError_t launch_expand_t_dtype(const SgmvArgs& a, hipStream_t stream) {
   switch ((a.d_in + 31) / 32) {
     case 1:
-      return launch_expand_t_ks<D, 1>(a, stream);
+      return launch_expand_t_ks<D, 1, kExpTLaneCols>(a, stream);
     case 2:
-      return launch_expand_t_ks<D, 2>(a, stream);
+      return launch_expand_t_ks<D, 2, kExpTLaneCols>(a, stream);
     case 3:
-      return launch_expand_t_ks<D, 3>(a, stream);
+      return launch_expand_t_ks<D, 3, kExpTLaneCols>(a, stream);
     case 4:
-      return launch_expand_t_ks<D, 4>(a, stream);
+      return launch_expand_t_ks<D, 4, kExpTLaneCols>(a, stream);
     default:
       return hipErrorInvalidValue;
   }
