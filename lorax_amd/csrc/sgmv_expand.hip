@@ -8,9 +8,10 @@
 // chunk of one segment:
 //   * long segments: the r x 64 panel of B goes through LDS once, every wave turns it
 //     into MFMA operands that stay in registers, and then walks 16-row blocks of the
-//     chunk computing the transposed product (B^T as the first MFMA operand, v as the
-//     second), which leaves each lane with 8 adjacent columns of one y row per pair of
-//     accumulators - y is read and written with 16-byte accesses and never staged;
+//     chunk computing v (first MFMA operand) times B (second).  Accumulator j stands for
+//     the columns 4c + j (c = lane & 15), which leaves each lane with 4 adjacent columns
+//     of the rows 4g .. 4g + 3 (g = lane >> 4): a y access of the wave is four whole
+//     128-byte runs, one per row, and y is never staged;
 //   * segments of a few rows (decode tokens inside a prefill batch): MFMA operand
 //     set-up would dominate, so the panel is streamed row by row on the vector ALU
 //     with 16-byte loads, each lane owning 8 adjacent columns.
@@ -18,7 +19,7 @@
 #include "sgmv_tiles.h"
 
 #ifndef LORAX_EXPAND_STAGES
-#define LORAX_EXPAND_STAGES 3
+#define LORAX_EXPAND_STAGES 2
 #endif
 
 namespace lorax {
@@ -30,12 +31,8 @@ constexpr int kExpandShortRows = 4;      // row tiles up to this height use the 
 constexpr int kPanelPitch = kExpandCols + 4;  // LDS row pitch in elements
 constexpr int kExpandStages = LORAX_EXPAND_STAGES;  // register stages of the row-block pipeline
 
-// Output column (0..63) that row `a` of the first MFMA operand of accumulator j
-// stands for.  Chosen so that lane group g = a / 4 ends up with columns
-// [8g, 8g+8) in accumulators 0,1 and [32+8g, 32+8g+8) in accumulators 2,3.
-__device__ __forceinline__ int panel_col(int j, int a) {
-  return (j >> 1) * 32 + (a >> 2) * 8 + (j & 1) * 4 + (a & 3);
-}
+// Output column (0..63) that column `c` of the second MFMA operand of accumulator j stands for.
+__device__ __forceinline__ int panel_col(int j, int c) { return 4 * c + j; }
 
 template <typename D, int KS>
 __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
@@ -110,14 +107,14 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
     }
 
     vec8 bf[4][KS];
+    typedef E yvec __attribute__((ext_vector_type(4)));
     const int nmb = (nrows + 15) / 16;
-    const bool col_ok0 = n0 + g * 8 < h_out;
-    const bool col_ok1 = n0 + 32 + g * 8 < h_out;
-    // Loads are unconditional: rows past the tile are clamped to its last row and columns past
-    // h_out to the panel's first vector (both valid memory); only the stores are predicated.
+    // h_out is a multiple of 8: a lane's four columns are inside the matrix or outside it as a whole.
+    // Loads are unconditional: rows past the tile are clamped to its last row and a lane past h_out
+    // reads the panel's first columns (both valid memory); only the stores are predicated.
     // v chunks beyond the rank are zeroed after the load.
-    const int coff0 = col_ok0 ? g * 8 : 0;
-    const int coff1 = col_ok1 ? 32 + g * 8 : 0;
+    const bool col_ok = n0 + 4 * c < h_out;
+    const int col = n0 + (col_ok ? 4 * c : 0);
     bool k_ok[KS];
     int k_off[KS];
 #pragma unroll
@@ -125,16 +122,18 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
       k_ok[s] = s * 32 + g * 8 < r;
       k_off[s] = k_ok[s] ? s * 32 + g * 8 : 0;
     }
-    auto load_block = [&](int mb, vec8(&vf)[KS], vec8& y0, vec8& y1) {
-      const int row = min(rt.row0 + mb * 16 + c, rt.row_end - 1);
-      const E* vp = V + static_cast<int64_t>(row) * r;
+    auto load_block = [&](int mb, vec8(&vf)[KS], yvec(&yv)[4]) {
+      const int vrow = min(rt.row0 + mb * 16 + c, rt.row_end - 1);
+      const E* vp = V + static_cast<int64_t>(vrow) * r;
 #pragma unroll
       for (int s = 0; s < KS; ++s) vf[s] = load8<D>(vp + k_off[s]);
-      const E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0;
-      y0 = load8<D>(yp + coff0);
-      y1 = load8<D>(yp + coff1);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = min(rt.row0 + mb * 16 + g * 4 + i, rt.row_end - 1);
+        yv[i] = *(const LORAX_GLOBAL yvec*)(Y + static_cast<int64_t>(row) * y_stride + y_offset + col);
+      }
     };
-    auto finish_block = [&](bool live, int mb, vec8(&vf)[KS], vec8 y0, vec8 y1) {
+    auto finish_block = [&](bool live, int mb, vec8(&vf)[KS], yvec(&yv)[4]) {
       f32x4 acc[4];
 #pragma unroll
       for (int s = 0; s < KS; ++s) vf[s] = keep_if<D>(k_ok[s], vf[s]);
@@ -142,22 +141,18 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
       for (int j = 0; j < 4; ++j) {
         acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < KS; ++s) acc[j] = D::mfma16(bf[j][s], vf[s], acc[j]);
+        for (int s = 0; s < KS; ++s) acc[j] = D::mfma16(vf[s], bf[j][s], acc[j]);
       }
-      const int row = rt.row0 + mb * 16 + c;
-      const bool ok = live && row < rt.row_end;
-      E* yp = Y + static_cast<int64_t>(row) * y_stride + y_offset + n0;
-      y0 = keep_if<D>(accumulate_into_y != 0, y0);  // overwrite mode: the old y counts as zero
-      y1 = keep_if<D>(accumulate_into_y != 0, y1);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        y0[i] = accumulate<D>(y0[i], acc[0][i]);
-        y0[4 + i] = accumulate<D>(y0[4 + i], acc[1][i]);
-        y1[i] = accumulate<D>(y1[i], acc[2][i]);
-        y1[4 + i] = accumulate<D>(y1[4 + i], acc[3][i]);
+        const int row = rt.row0 + mb * 16 + g * 4 + i;
+        yvec out;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)  // overwrite mode: the old y counts as zero
+          out[j] = accumulate<D>(accumulate_into_y != 0 ? yv[i][j] : static_cast<E>(0.0f), acc[j][i]);
+        if (live && col_ok && row < rt.row_end)
+          *(LORAX_GLOBAL yvec*)(Y + static_cast<int64_t>(row) * y_stride + y_offset + col) = out;
       }
-      if (ok && col_ok0) store8<D>(yp + g * 8, y0);
-      if (ok && col_ok1) store8<D>(yp + 32 + g * 8, y1);
     };
 
     // This wave's 16-row blocks are wave, wave + 4, ... below nmb.  They run through a ring of
@@ -168,9 +163,10 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
     // not depend on it, so the tile's first memory round trip overlaps the operand set-up.
     const int n = wave < nmb ? (nmb - wave + kExpandWaves - 1) / kExpandWaves : 0;
     auto block_of = [&](int i) { return wave + min(i, max(n, 1) - 1) * kExpandWaves; };
-    vec8 vr[kExpandStages][KS], y0r[kExpandStages], y1r[kExpandStages];
+    vec8 vr[kExpandStages][KS];
+    yvec yr[kExpandStages][4];
 #pragma unroll
-    for (int s = 0; s < kExpandStages - 1; ++s) load_block(block_of(s), vr[s], y0r[s], y1r[s]);
+    for (int s = 0; s < kExpandStages - 1; ++s) load_block(block_of(s), vr[s], yr[s]);
 
     // ---- MFMA path ----
     // Stage the r x 64 panel of B in LDS (rows k >= r and columns >= h_out as zeros).
@@ -201,10 +197,9 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
 #pragma unroll
         for (int s = 0; s < kExpandStages; ++s) {
           constexpr int kAhead = kExpandStages - 1;
-          load_block(block_of(i + s + kAhead), vr[(s + kAhead) % kExpandStages], y0r[(s + kAhead) % kExpandStages],
-                     y1r[(s + kAhead) % kExpandStages]);
+          load_block(block_of(i + s + kAhead), vr[(s + kAhead) % kExpandStages], yr[(s + kAhead) % kExpandStages]);
           __builtin_amdgcn_sched_barrier(0);
-          finish_block(i + s < n, block_of(i + s), vr[s], y0r[s], y1r[s]);
+          finish_block(i + s < n, block_of(i + s), vr[s], yr[s]);
         }
       }
     }
