@@ -176,7 +176,8 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
  *   accumulate = 1 is the reference's only mode; accumulate = 0 stores dtype(v @ B) into the rows of the
  *   segments instead of adding it (add_inputs=False of lorax_server/utils/ops/sgmv_expand.py:106-121).
  *
- * r must be a multiple of 8 in [8, 128]; h_out, y_offset and y_stride multiples of 8.
+ * r must be a multiple of 8 in [8, 128]; h_out, y_offset and y_stride multiples of 8; y_stride < 2^24
+ * (a row tile of y is addressed with 32-bit element offsets).
  */
 int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,

@@ -276,6 +276,8 @@ int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32
   if (y_offset < 0 || y_offset % 8 != 0 || y_stride % 8 != 0 || y_stride < y_offset + h_out)
     return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld must be multiples of 8 holding h_out=%d columns",
                 (long long)y_offset, (long long)y_stride, h_out);
+  if (y_stride >= (1ll << 24))
+    return fail(LORAX_EINVAL, "y_stride=%lld: rows of y hold fewer than 2^24 elements", (long long)y_stride);
   SgmvArgs a{};
   a.y = y;
   a.x = v;

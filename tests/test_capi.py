@@ -83,6 +83,8 @@ def test_sgmv_expand_validation():
             assert f(P, P, P, P, P, 2, 16, r, h, layout, 0, h, 0, 1, P, 120, 1, None) == ENOKERNEL, (r, h)
         assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 4, 8192, 0, 1, P, 120, 1, None) == EINVAL  # unaligned window
         assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 4096, 4096, 0, 1, P, 120, 1, None) == EINVAL  # too wide
+        assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 0, 1 << 24, 0, 1, P, 120, 1, None) == EINVAL  # row pitch
+        assert "2^24" in _err()
     assert f(P, P, P, P, P, 2, 16, 16, 4096, 2, 0, 4096, 0, 1, P, 120, 1, None) == EINVAL  # unknown layout
 
 
