@@ -80,6 +80,7 @@ class LoraLinear(nn.Module):
         columns [start, end) of `result`."""
         tensor_parallel = self.process_group.size() > 1
         decode_jobs = defaultdict(list)  # rank -> [(rank_segments, start, width)]
+        stacked_jobs = []  # (lora_a_stack, lora_b_stack, start, width) of projections served by stacked weights
         for name, start, end in slices:
             data = self._lora_data(adapter_data, name)
             if data is None:
@@ -94,13 +95,8 @@ class LoraLinear(nn.Module):
                 and key in adapter_data.layer_to_lora_weights
                 and input.shape[0] <= wrapper.max_batch_size
             ):
-                whole = end - start == result.shape[1]
                 lora_a_weights, lora_b_weights = adapter_data.layer_to_lora_weights[key]
-                wrapper.add_lora(
-                    result, input, lora_a_weights, lora_b_weights, 1.0,
-                    None if whole else start, None if whole else end - start,
-                    callback=self.collect_lora_a if tensor_parallel else None,
-                )
+                stacked_jobs.append((lora_a_weights, lora_b_weights, start, end - start))
                 continue
             sliced = end - start != result.shape[1]
             for r, rs in data.rank_data.items():
@@ -137,6 +133,11 @@ class LoraLinear(nn.Module):
                     lora_b_sgmv_cutlass(
                         result, v, rs.tmp_expand, rs.lora_b_ptr, rs.segment_starts, rs.segment_ends, self.layer_id
                     )
+
+        if stacked_jobs:  # the reference calls add_lora once per projection (utils/layers.py:92-104)
+            adapter_data.punica_wrapper.add_lora_slices(
+                result, input, stacked_jobs, 1.0, callback=self.collect_lora_a if tensor_parallel else None
+            )
 
         # Decode.  When every job of the call has a small A slab (rank 8 or 16, moderate widths), shrink and
         # expand run in one launch per rank and v never leaves the chip.  Otherwise all rank groups of all

@@ -1,5 +1,6 @@
 """The six LoRA operators of lorax_server/utils/ops (bgmv_shrink / bgmv_expand / bgmv_expand_slice /
-sgmv_shrink / sgmv_expand / sgmv_expand_slice) on the HIP kernels of this package.
+sgmv_shrink / sgmv_expand / sgmv_expand_slice) on the HIP kernels of this package, plus bgmv_lora_slices,
+which runs the decode update of several column slices in two launches.
 
 Same names, argument orders and meaning as the reference's Triton operators, which index ONE stacked
 weight tensor per layer - lora_a_weights [num_loras, r, h_in], lora_b_weights [num_loras, h_out, r], an
@@ -151,6 +152,45 @@ def bgmv_expand(
     width = lora_b_weights.size(-2)
     assert output_tensor.size(1) == width
     bgmv_expand_slice(inputs, lora_b_weights, output_tensor, lora_indices_tensor, 0, width, add_inputs)
+
+
+@torch.inference_mode()
+def bgmv_lora_slices(
+    inputs: torch.Tensor,
+    slices,
+    output_tensor: torch.Tensor,
+    lora_indices_tensor: torch.Tensor,
+    scaling: float = 1.0,
+):
+    """bgmv_shrink followed by bgmv_expand_slice(add_inputs=True) for several column slices of output_tensor that
+    share `inputs` (q/k/v, gate/up): `slices` is a sequence of (lora_a_weights, lora_b_weights, slice_offset,
+    slice_size), ranks may differ.  No counterpart among the reference's operators, which its wrapper calls once
+    per slice (punica.py:750-773); here the shrinks of up to 16 slices are one launch and their expands another,
+    and the intermediate is kept in the type of `inputs` and never zero-filled (the shrink overwrites the rows
+    of routed tokens and the expand reads no others)."""
+    assert inputs.dtype in (torch.float16, torch.bfloat16)
+    assert inputs.is_contiguous() and output_tensor.is_contiguous()
+    assert inputs.size(0) == output_tensor.size(0)
+    jobs = []
+    for lora_a_weights, lora_b_weights, slice_offset, slice_size in slices:
+        a = _stacked(lora_a_weights, "lora_a_weights")
+        b = _stacked(lora_b_weights, "lora_b_weights")
+        assert a.dtype == inputs.dtype and b.dtype == inputs.dtype
+        assert inputs.size(1) == a.size(-1) and a.size(-2) == b.size(-1) and slice_size == b.size(-2)
+        jobs.append((stack_table(a), stack_table(b), a.size(-2), slice_offset, slice_size))
+    step = _native.MAX_BGMV_PROBLEMS
+    tokens = inputs.size(0)
+    for i in range(0, len(jobs), step):
+        chunk = jobs[i : i + step]
+        flat = torch.empty((tokens * sum(r for _, _, r, _, _ in chunk),), dtype=inputs.dtype, device=inputs.device)
+        bufs, pos = [], 0
+        for _, _, r, _, _ in chunk:
+            bufs.append(flat[pos : pos + tokens * r].view(tokens, r))
+            pos += tokens * r
+        _native.bgmv_multi([(v, inputs, ta, lora_indices_tensor, 0, None) for v, (ta, _, _, _, _) in zip(bufs, chunk)],
+                           0, scaling, False)
+        _native.bgmv_multi([(output_tensor, v, tb, lora_indices_tensor, off, size)
+                            for v, (_, tb, _, off, size) in zip(bufs, chunk)], 0, 1.0, True)
 
 
 @torch.inference_mode()

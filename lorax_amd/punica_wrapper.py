@@ -192,6 +192,25 @@ class PunicaWrapper:
             self.add_expand_slice(y, buffer, wb_t_all, y_offset, y_slice_size, add_input=True)
         y = y.view_as(y_org)
 
+    def add_lora_slices(self, y: torch.Tensor, x: torch.Tensor, slices, scale: float,
+                        callback: Optional[Callable] = None) -> None:
+        """add_lora for several column slices of y that share x; `slices` is a sequence of
+        (wa_t_all, wb_t_all, y_offset, y_slice_size).  In decode, without a callback between shrink and expand,
+        all shrinks are one launch and all expands another; otherwise one add_lora per slice."""
+        if not slices:
+            return
+        y2 = y.view(-1, y.shape[-1])
+        x2 = x.view(-1, x.shape[-1])
+        batched = (not self.is_prefill and callback is None and x2.dtype in (torch.float16, torch.bfloat16)
+                   and all(wa.dtype == x2.dtype and wb.dtype == x2.dtype for wa, wb, _, _ in slices))
+        if batched:
+            ops.bgmv_lora_slices(x2, slices, y2, self.token_lora_indices, scale)
+            return
+        for wa_t_all, wb_t_all, y_offset, y_slice_size in slices:
+            whole = y_offset == 0 and y_slice_size == y2.shape[1]
+            self.add_lora(y2, x2, wa_t_all, wb_t_all, scale, None if whole else y_offset,
+                          None if whole else y_slice_size, callback=callback)
+
     def add_lora_packed_nslice(
         self,
         y: torch.Tensor,
@@ -202,15 +221,11 @@ class PunicaWrapper:
         output_slices: Tuple[int, ...],
     ) -> None:
         """add_lora for every slice of a packed projection (q/k/v, gate/up), punica.py:750-773."""
-        y_org = y
-        x = x.view(-1, x.shape[-1])
-        y = y.view(-1, y.shape[-1])
-        offset_left = 0
+        slices, offset_left = [], 0
         for slice_idx in range(len(output_slices)):
-            self.add_lora(y, x, lora_a_stacked[slice_idx], lora_b_stacked[slice_idx], scale, offset_left,
-                          output_slices[slice_idx])
+            slices.append((lora_a_stacked[slice_idx], lora_b_stacked[slice_idx], offset_left, output_slices[slice_idx]))
             offset_left += output_slices[slice_idx]
-        y = y.view_as(y_org)
+        self.add_lora_slices(y, x, slices, scale)
 
     def add_lora_logits(
         self,
