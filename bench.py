@@ -66,7 +66,8 @@ class Plan:
 
     pattern "fused" is what lorax_amd.layers issues: in decode one batched shrink launch and one batched
     expand launch per projection group and rank (the shrink overwrites v, no zero-fill); in prefill a
-    zero-fill, a shrink and an expand per projection and rank.  pattern "reference" is the reference
+    zero-fill and a shrink per projection group and rank (up to a summed rank of 128 per launch) and an
+    expand per projection and rank.  pattern "reference" is the reference
     caller's sequence (utils/layers.py:114-164): zero-fill, shrink, expand for every projection and rank.
     """
 
@@ -95,13 +96,25 @@ class Plan:
                         jobs.append((data.use_sgmv, r, rd, off, size))
                 off += size
             decode = defaultdict(list)
+            prefill = defaultdict(list)  # (rank, segment tables) -> [(rank_segments, offset, width)]
             for use_sgmv, r, rd, off, size in jobs:
                 if use_sgmv:
-                    self._add_sgmv(x, y, off, size, group.h_in, r, rd)
+                    from lorax_amd import sgmv
+
+                    if (pattern == "fused" and rd.segments_key is not None
+                            and sgmv.resident_shrink_applies(r, group.h_in, T)):
+                        prefill[(r, rd.segments_key)].append((rd, off, size))
+                    else:
+                        self._add_sgmv(x, y, off, size, group.h_in, r, rd)
                 elif pattern == "reference":
                     self._add_bgmv_reference(x, y, off, size, group.h_in, r, rd)
                 else:
                     decode[r].append((rd, off, size))
+            # as lorax_amd.layers: projections of one rank and the same segment tables shrink in one launch
+            for (r, _), same in prefill.items():
+                step = max(1, min(_native.MAX_SGMV_SHRINK_PROBLEMS, 128 // r))
+                for i in range(0, len(same), step):
+                    self._add_sgmv_group(x, y, group.h_in, r, same[i:i + step])
             all_jobs = [(r, rd, off, size) for r, rank_jobs in decode.items() for rd, off, size in rank_jobs]
             all_fused = bool(all_jobs) and self.use_plan and self.fuse_small_ranks and all(
                 _native.bgmv_lora_fits(r, group.h_in, size) for r, _, _, size in all_jobs)
@@ -159,6 +172,40 @@ class Plan:
                            2 * rows * r * h_in))
         self.calls.append(("sgmv_expand", expand, rows * r * e + uniq * r * size * e + 2 * rows * size * e,
                            2 * rows * r * size))
+
+    def _add_sgmv_group(self, x, y, h_in, r, jobs):
+        """Zero-fill and shrink of up to four projections in one launch each (x counted once), then one
+        expand per projection from the resident B^T stacks."""
+        import torch
+
+        from lorax_amd import _native, sgmv
+
+        e = 2
+        first = jobs[0][0]
+        starts, ends = first.segment_starts, first.segment_ends
+        lens = (ends - starts).clamp(min=0)
+        rows = int(lens.sum().item())
+        flat = torch.zeros((len(jobs), x.size(0), r), dtype=x.dtype, device=x.device)
+        vs = list(flat.unbind(0))
+        tables = [rd.lora_a_t_ptr for rd, _, _ in jobs]
+        tmp_s = sgmv.get_tmp_tensor(x.device)
+        shrink_bytes = rows * h_in * e
+        for rd, _, _ in jobs:
+            uniq = len(set(rd.lora_a_t_ptr[lens > 0].tolist()))
+            shrink_bytes += uniq * r * h_in * e + rows * r * e
+        self.calls.append(("zero", lambda layer: flat.zero_(), 0, 0))
+        self.calls.append(("sgmv_shrink",
+                           lambda layer: _native.sgmv_shrink_multi(vs, x, tables, starts, ends, tmp_s, layer),
+                           shrink_bytes, 2 * rows * r * h_in * len(jobs)))
+        for v, (rd, off, size) in zip(vs, jobs):
+            uniq = len(set(rd.lora_b_t_ptr[lens > 0].tolist()))
+
+            def expand(layer, v=v, rd=rd, off=off, size=size):
+                sgmv.lora_b_sgmv_cutlass_slice(y, v, rd.tmp_expand, rd.lora_b_t_ptr, rd.segment_starts,
+                                               rd.segment_ends, layer, off, size, transposed=True)
+
+            self.calls.append(("sgmv_expand", expand, rows * r * e + uniq * r * size * e + 2 * rows * size * e,
+                               2 * rows * r * size))
 
     def _add_bgmv_reference(self, x, y, off, size, h_in, r, rd):
         import torch

@@ -166,6 +166,25 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
                       void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
 
 /*
+ * SGMV shrink of up to 4 projections that share x, the segments and the rank (q/k/v, gate/up), LORAX_A_RH
+ * stacks: problem p gets v_p[s:e, :] += dtype(scale * x[s:e, :] @ A_p^T) exactly as from lorax_sgmv_shrink
+ * with (v_p, w_ptrs_p).  The reference launches one shrink per projection (lorax_server/utils/layers.py:
+ * 121-133, punica_ops.cc:369-411) and reads x once per launch; here, when num_problems * r <= 128, h_in is a
+ * multiple of 128 and the batch has more than 512 rows, the projections run as ONE launch that reads x once
+ * (their A matrices are stacked into one rank-(num_problems * r) tile).  Otherwise the call issues one
+ * launch per projection.  `tmp`/`tmp_bytes` as for lorax_sgmv_shrink with LORAX_A_RH.
+ */
+typedef struct {
+  void* v;               /* [num_tokens, r] */
+  const int64_t* w_ptrs; /* [num_segments] addresses of [num_layers, r, h_in] stacks */
+} lorax_sgmv_shrink_problem_t;
+
+int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t num_problems, const void* x,
+                            const int32_t* s_start, const int32_t* s_end, int32_t num_segments,
+                            int64_t num_tokens, int32_t h_in, int32_t r, int64_t layer_idx, float scale,
+                            void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
+
+/*
  * SGMV expand.  Replaces the expand direction of sgmv_cutlass (punica_ops.cc:338-367,
  * sgmv/sgmv_cutlass.cuh:86-131).
  *

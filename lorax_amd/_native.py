@@ -42,6 +42,12 @@ class BgmvProblem(ctypes.Structure):
     ]
 
 
+class SgmvShrinkProblem(ctypes.Structure):
+    """lorax_sgmv_shrink_problem_t of include/lorax_hip.h."""
+
+    _fields_ = [("v", _c.c_void_p), ("w_ptrs", _c.c_void_p)]
+
+
 class AdapterEntry(ctypes.Structure):
     """lorax_adapter_entry_t of include/lorax_hip.h."""
 
@@ -82,6 +88,11 @@ _SIGNATURES = {
         [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
          _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_void_p, _c.c_int64, _c.c_int32,
          _c.c_void_p],
+    ),
+    "lorax_sgmv_shrink_multi": (
+        _c.c_int,
+        [_c.POINTER(SgmvShrinkProblem), _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
+         _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_void_p, _c.c_int64, _c.c_int32, _c.c_void_p],
     ),
     "lorax_sgmv_expand": (
         _c.c_int,
@@ -390,6 +401,34 @@ def sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, scale: float = 1.0)
     if isinstance(tmp, torch.Tensor) and tmp.dtype != torch.uint8:
         raise RuntimeError(f"CHECK_EQ(tmp.scalar_type(), at::ScalarType::Byte) failed. {tmp.dtype}")
     return _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, A_RH, scale)
+
+
+MAX_SGMV_SHRINK_PROBLEMS = 4
+
+
+def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: float = 1.0) -> None:
+    """lorax_sgmv_shrink_multi: sgmv_shrink for up to 4 projections (outputs `ys`, pointer tables `w_ptrs`) that
+    share x, the segment tables and the rank; one launch that reads x once where the kernels allow it."""
+    if not 1 <= len(ys) <= MAX_SGMV_SHRINK_PROBLEMS or len(ys) != len(w_ptrs):
+        raise RuntimeError(f"between 1 and {MAX_SGMV_SHRINK_PROBLEMS} outputs with one pointer table each")
+    if isinstance(tmp, torch.Tensor) and tmp.dtype != torch.uint8:
+        raise RuntimeError(f"CHECK_EQ(tmp.scalar_type(), at::ScalarType::Byte) failed. {tmp.dtype}")
+    arr = (SgmvShrinkProblem * len(ys))()
+    for i, (y, w_ptr) in enumerate(zip(ys, w_ptrs)):
+        _check_sgmv(y, x, w_ptr, s_start, s_end, tmp)
+        if y.size(1) != ys[0].size(1):
+            raise RuntimeError("the projections of one call share the rank")
+        arr[i] = SgmvShrinkProblem(y.data_ptr(), w_ptr.data_ptr())
+    if not torch.cuda.is_current_stream_capturing():
+        init(x.device)
+    with torch.cuda.device(x.device):
+        rc = lib().lorax_sgmv_shrink_multi(
+            arr, len(ys), x.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0), x.size(0), x.size(1),
+            ys[0].size(1), int(layer_idx), float(scale), tmp.data_ptr(), tmp.numel() * tmp.element_size(),
+            _dtype_code(x), _stream(x),
+        )
+    if rc != 0:
+        _raise_last(rc)
 
 
 ESPACE = 5

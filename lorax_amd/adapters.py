@@ -174,7 +174,7 @@ class RankSegments:
                  tmp_expand: Optional[torch.Tensor], segment_starts: Optional[torch.Tensor],
                  segment_ends: Optional[torch.Tensor], indices: Optional[torch.Tensor],
                  plan: Optional[torch.Tensor] = None, lora_a_t_ptr: Optional[torch.Tensor] = None,
-                 lora_b_t_ptr: Optional[torch.Tensor] = None):
+                 lora_b_t_ptr: Optional[torch.Tensor] = None, segments_key=None):
         self.rank = rank
         self._lora_a_ptr = lora_a_ptr  # a tensor, or a function that builds it
         self._lora_b_ptr = lora_b_ptr
@@ -193,6 +193,9 @@ class RankSegments:
         # prefill: addresses of the resident stacks, one per segment like lora_a_ptr / lora_b_ptr
         self.lora_a_t_ptr = lora_a_t_ptr
         self.lora_b_t_ptr = lora_b_t_ptr
+        # prefill: hashable and equal for rank groups (of different layer types) whose segment_starts /
+        # segment_ends hold the same values - their shrinks can share one pass over x; None = unknown
+        self.segments_key = segments_key
 
     @property
     def lora_a_ptr(self) -> Optional[torch.Tensor]:
@@ -398,6 +401,7 @@ class BatchLoraWeights(BatchAdapterWeights):
                 plan=plan,
                 lora_a_t_ptr=lora_a_t_ptr[segs] if use_sgmv else None,
                 lora_b_t_ptr=lora_b_t_ptr[segs] if use_sgmv else None,
+                segments_key=(tuple(segs), head_starts is not None) if use_sgmv else None,
             )
 
         return cls(
@@ -627,6 +631,8 @@ def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAda
                     indices=None,
                     lora_a_t_ptr=a_ptr,
                     lora_b_t_ptr=b_ptr,
+                    segments_key=(packed[g.starts_off : g.starts_off + 4 * n].tobytes(),
+                                  packed[g.ends_off : g.ends_off + 4 * n].tobytes()),
                 )
             else:
                 rank_data[g.rank] = RankSegments(

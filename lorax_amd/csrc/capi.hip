@@ -251,6 +251,64 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
   return LORAX_OK;
 }
 
+int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t num_problems, const void* x,
+                            const int32_t* s_start, const int32_t* s_end, int32_t num_segments,
+                            int64_t num_tokens, int32_t h_in, int32_t r, int64_t layer_idx, float scale,
+                            void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
+  if (num_problems < 1 || num_problems > kMaxShrinkGroup)
+    return fail(LORAX_EINVAL, "num_problems=%d (1 to %d per call)", num_problems, kMaxShrinkGroup);
+  if (problems == nullptr) return fail(LORAX_EINVAL, "null pointer argument (problems)");
+  // One launch where the LDS-staged kernel takes the stacked rank and the batch is past the streaming
+  // kernel's range; otherwise one launch per projection, with the same result.
+  const int rows_max = tuning().shrink_rows_max != 0 ? tuning().shrink_rows_max : 512;
+  const bool stacked = num_problems > 1 && r >= 8 && r % 8 == 0 && num_problems * r <= kMaxRank && h_in > 0 &&
+                       h_in % 128 == 0 && num_tokens > rows_max && tuning().shrink_lds >= 0;
+  if (!stacked) {
+    for (int i = 0; i < num_problems; ++i) {
+      const int rc = lorax_sgmv_shrink(problems[i].v, x, problems[i].w_ptrs, s_start, s_end, num_segments, num_tokens,
+                                       h_in, r, LORAX_A_RH, layer_idx, scale, tmp, tmp_bytes, dtype, stream);
+      if (rc != LORAX_OK) return rc;
+    }
+    return LORAX_OK;
+  }
+  if (num_segments < 0 || num_tokens < 0)
+    return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments, (long long)num_tokens);
+  if (tmp_bytes != LORAX_SHRINK_TMP_BYTES)
+    return fail(LORAX_ETMPSIZE, "CHECK_EQ(tmp.size(0), 8 * 1024 * 1024) failed. %lld vs %d", (long long)tmp_bytes,
+                LORAX_SHRINK_TMP_BYTES);
+  if (num_segments == 0) return LORAX_OK;
+  for (int i = 0; i < num_problems; ++i)
+    if (int rc = check_common(problems[i].v, x, problems[i].w_ptrs, dtype)) return rc;
+  if (s_start == nullptr || s_end == nullptr || tmp == nullptr)
+    return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p tmp=%p)", s_start, s_end, tmp);
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  if (num_tokens > INT32_MAX / 2)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in, r, LORAX_A_RH);
+  SgmvArgs a{};
+  a.y = problems[0].v;
+  a.x = x;
+  a.w_ptrs = problems[0].w_ptrs;
+  a.s_start = s_start;
+  a.s_end = s_end;
+  a.num_segments = num_segments;
+  a.num_tokens = num_tokens;
+  a.d_in = h_in;
+  a.d_out = num_problems * r;
+  a.a_layout = LORAX_A_RH;
+  a.layer_idx = layer_idx;
+  a.dtype = dtype;
+  a.scale = scale;
+  a.group.count = num_problems;
+  a.group.rank = r;
+  for (int i = 0; i < num_problems; ++i) {
+    a.group.v[i] = problems[i].v;
+    a.group.w[i] = problems[i].w_ptrs;
+  }
+  const hipError_t e = launch_sgmv_shrink_lds(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_shrink launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
 int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
                       int32_t h_out, int32_t b_layout, int64_t y_offset, int64_t y_stride,

@@ -61,6 +61,16 @@ struct BgmvArgs {
   int dtype;
 };
 
+// Projections that share x, the segment tables and the rank, shrunk in one launch (the LDS-staged kernel
+// treats them as one problem whose rank is the sum): outputs and pointer tables per projection.
+constexpr int kMaxShrinkGroup = 4;
+struct ShrinkGroup {
+  void* v[kMaxShrinkGroup];
+  const int64_t* w[kMaxShrinkGroup];
+  int count;
+  int rank;  // of each projection
+};
+
 struct SgmvArgs {
   void* y;        // v for shrink, y for expand
   const void* x;  // x for shrink, v for expand
@@ -76,6 +86,7 @@ struct SgmvArgs {
   int64_t y_stride;
   int64_t layer_idx;
   int dtype;
+  ShrinkGroup group;  // shrink of several projections: count > 1, d_out = count * rank; else unused
   float scale;     // shrink: factor applied to the fp32 sums before rounding (1 in the reference's calls)
   int accumulate;  // expand: 1 = add to y (the reference's only mode), 0 = overwrite the rows of the segments
   // library workspace of the current device (shrink split-K)

@@ -56,14 +56,16 @@ __device__ __forceinline__ void wait_pending(int pending) {
 
 template <typename D, int NB, int MBLK, bool KSPLIT>
 __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
-    typename D::E* __restrict__ V, const typename D::E* __restrict__ X,
-    const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
-    const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int r,
-    int64_t layer_idx, int stages, float scale) {
+    const ShrinkGroup grp, const typename D::E* __restrict__ X, const int32_t* __restrict__ s_start,
+    const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int64_t layer_idx,
+    int stages, float scale) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
-  // NB = ceil(r / 16) rank blocks; the rank itself only needs to be a multiple of 8: rows of the A tile past
-  // the rank re-read the last row and their columns of the result are not stored.
+  // The A tile stacks the A matrices of grp.count projections of rank r: row p * r + i is row i of
+  // projection p, and column p * r + i of the result goes to projection p's v.  (One projection: the
+  // plain shrink.)  NB = ceil(count * r / 16) rank blocks; r only needs to be a multiple of 8: rows of the
+  // A tile past count * r re-read the last row and their columns of the result are not stored.
+  const int r = grp.rank;
   constexpr int R = NB * 16;
   constexpr int ROWS = MBLK * 16;
   constexpr int kXBytes = ROWS * kLdsRowBytes;
@@ -97,7 +99,10 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
   for (int tile = vb.x;; tile += gridDim.x) {
     RowTile rt;
     if (!find_row_tile(s_start, s_end, num_segments, num_tokens, ROWS, tile, rt)) break;
-    const E* A = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * r * static_cast<int64_t>(h_in);
+    const E* A[kMaxShrinkGroup];
+#pragma unroll
+    for (int p = 0; p < kMaxShrinkGroup; ++p)
+      A[p] = reinterpret_cast<const E*>(grp.w[p < grp.count ? p : 0][rt.seg]) + layer_idx * r * static_cast<int64_t>(h_in);
 
     // Source addresses of this thread's chunks.  Load j of a thread covers chunk id j * 256 + tid of
     // the tile: row = id / 16, position = id % 16, and it fetches the row's chunk position ^ (row & 15).
@@ -114,7 +119,10 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     for (int j = 0; j < kALoads; ++j) {
       const int id = j * kLdsThreads + tid;
       const int row = id >> 4;
-      asrc[j] = A + static_cast<int64_t>(min(row, r - 1)) * h_in + (((id & 15) ^ (row & 15)) << 3);
+      int proj = row / r, arow = row - proj * r;
+      if (proj >= grp.count) proj = grp.count - 1, arow = r - 1;
+      const E* Ap = proj == 0 ? A[0] : (proj == 1 ? A[1] : (proj == 2 ? A[2] : A[3]));
+      asrc[j] = Ap + static_cast<int64_t>(arow) * h_in + (((id & 15) ^ (row & 15)) << 3);
     }
     auto issue = [&](int st, int slot) {
       char* buf = lds + slot * kStageBytes;
@@ -171,6 +179,14 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     }
 
     // acc[mb][nb][i] of lane (g, c) is D[n = nblock*16 + 4g + i][row = mblock*16 + c].
+    // Four adjacent columns of one row (r is a multiple of 8: they belong to one projection).
+    auto store4 = [&](int row, int col, f32x4 sum) {
+      const int proj = col / r;
+      if (row < rt.row_end && proj < grp.count) {
+        E* Vp = static_cast<E*>(proj == 0 ? grp.v[0] : (proj == 1 ? grp.v[1] : (proj == 2 ? grp.v[2] : grp.v[3])));
+        accumulate4<D>(Vp + static_cast<int64_t>(row) * r + (col - proj * r), sum * scale);
+      }
+    };
     if constexpr (KSPLIT) {
       // Partial sums of the four waves meet in LDS (the stage buffers are free: the last stage was
       // waited for with no load outstanding), then the 256 threads share the blocks' elements.
@@ -191,7 +207,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
         }
         const int row = rt.row0 + (blk / NB) * 16 + (l & 15);
         const int col = (blk % NB) * 16 + 4 * (l >> 4);
-        if (row < rt.row_end && col < r) accumulate4<D>(V + static_cast<int64_t>(row) * r + col, sum * scale);
+        store4(row, col, sum);
       }
     } else {
       // every wave owns its output blocks: no cross-wave reduction
@@ -202,7 +218,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
 #pragma unroll
           for (int nb = 0; nb < NPW; ++nb) {
             const int col = (wn * NPW + nb) * 16 + 4 * g;
-            if (col < r) accumulate4<D>(V + static_cast<int64_t>(row) * r + col, acc[mb][nb] * scale);
+            store4(row, col, acc[mb][nb]);
           }
         }
       }
@@ -240,9 +256,17 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
     if (device >= 0 && device < 64) configured[device] = true;
   }
   dim3 grid(static_cast<unsigned>(tiles < (1 << 20) ? tiles : (1 << 20)));
-  hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, static_cast<typename D::E*>(a.y),
-                     static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end, a.num_segments,
-                     static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, stages, a.scale);
+  ShrinkGroup grp = a.group;
+  if (grp.count <= 1) {
+    grp = ShrinkGroup{};
+    grp.v[0] = a.y;
+    grp.w[0] = a.w_ptrs;
+    grp.count = 1;
+    grp.rank = a.d_out;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, grp, static_cast<const typename D::E*>(a.x),
+                     a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages,
+                     a.scale);
   return hipGetLastError();
 }
 

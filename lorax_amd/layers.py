@@ -27,11 +27,14 @@ from torch import nn
 
 from lorax_amd import _native
 from lorax_amd.adapters import LORA, AdapterBatchData, BatchLoraWeights
+from lorax_amd._native import MAX_SGMV_SHRINK_PROBLEMS
 from lorax_amd.sgmv import (
+    MAX_RANK_CUSTOM,
     get_tmp_tensor,
     has_sgmv,
     lora_a_sgmv_cutlass,
     lora_a_sgmv_resident,
+    lora_a_sgmv_resident_multi,
     lora_b_sgmv_cutlass,
     lora_b_sgmv_cutlass_slice,
     resident_shrink_applies,
@@ -81,6 +84,7 @@ class LoraLinear(nn.Module):
         tensor_parallel = self.process_group.size() > 1
         decode_jobs = defaultdict(list)  # rank -> [(rank_segments, start, width)]
         stacked_jobs = []  # (lora_a_stack, lora_b_stack, start, width) of projections served by stacked weights
+        prefill_jobs = defaultdict(list)  # (rank, segment tables) -> [(rank_segments, start, width)]
         for name, start, end in slices:
             data = self._lora_data(adapter_data, name)
             if data is None:
@@ -109,6 +113,9 @@ class LoraLinear(nn.Module):
                 # the reference's prefill layouts are only touched for shapes the resident-layout shrink
                 # does not take.
                 if rs.lora_a_t_ptr is not None and resident_shrink_applies(r, input.size(1), input.size(0)):
+                    if rs.segments_key is not None and rs.lora_b_t_ptr is not None and not tensor_parallel:
+                        prefill_jobs[(r, rs.segments_key)].append((rs, start, end - start))
+                        continue
                     v = lora_a_sgmv_resident(
                         input, get_tmp_tensor(input.device), rs.lora_a_t_ptr, rs.segment_starts, rs.segment_ends,
                         self.layer_id, r,
@@ -132,6 +139,24 @@ class LoraLinear(nn.Module):
                 else:
                     lora_b_sgmv_cutlass(
                         result, v, rs.tmp_expand, rs.lora_b_ptr, rs.segment_starts, rs.segment_ends, self.layer_id
+                    )
+
+        # Prefill: projections of one rank with the same segment tables (q/k/v, gate/up of adapters that target
+        # them all) shrink together, as many per launch as fit a summed rank of 128 - x is read once per
+        # launch; the reference issues one shrink per projection (utils/layers.py:121-133).
+        for (r, _), group in prefill_jobs.items():
+            step = max(1, min(MAX_SGMV_SHRINK_PROBLEMS, MAX_RANK_CUSTOM // r))
+            for i in range(0, len(group), step):
+                chunk = group[i : i + step]
+                first = chunk[0][0]
+                vs = lora_a_sgmv_resident_multi(
+                    input, get_tmp_tensor(input.device), [rs.lora_a_t_ptr for rs, _, _ in chunk],
+                    first.segment_starts, first.segment_ends, self.layer_id, r,
+                )
+                for v, (rs, start, width) in zip(vs, chunk):
+                    lora_b_sgmv_cutlass_slice(
+                        result, v, rs.tmp_expand, rs.lora_b_t_ptr, rs.segment_starts, rs.segment_ends,
+                        self.layer_id, start, width, transposed=True,
                     )
 
         if stacked_jobs:  # the reference calls add_lora once per projection (utils/layers.py:92-104)

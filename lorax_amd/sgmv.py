@@ -14,7 +14,7 @@ plain PyTorch.
 import os
 import warnings
 from functools import lru_cache
-from typing import List, Optional, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 import torch.nn.functional as F
@@ -147,6 +147,24 @@ def lora_a_sgmv_resident(
     v = torch.zeros((x.size(0), lora_rank), dtype=x.dtype, device=x.device)
     _native_module().sgmv_shrink(v, x, wa_t_ptr, s_start, s_end, tmp, layer_idx)
     return v
+
+
+def lora_a_sgmv_resident_multi(
+    x: torch.Tensor,
+    tmp: torch.Tensor,
+    wa_t_ptrs: Sequence[torch.Tensor],
+    s_start: torch.IntTensor,
+    s_end: torch.IntTensor,
+    layer_idx: int,
+    lora_rank: int,
+) -> List[torch.Tensor]:
+    """lora_a_sgmv_resident for up to 4 projections that share x, the segments and the rank (q/k/v, gate/up):
+    one v per pointer table.  One launch that reads x once when the summed rank is at most 128 and h_in a
+    multiple of 128; the reference issues one shrink per projection (layers.py:121-133)."""
+    flat = torch.zeros((len(wa_t_ptrs), x.size(0), lora_rank), dtype=x.dtype, device=x.device)
+    vs = list(flat.unbind(0))
+    _native_module().sgmv_shrink_multi(vs, x, list(wa_t_ptrs), s_start, s_end, tmp, layer_idx)
+    return vs
 
 
 def resident_shrink_applies(lora_rank: int, h_in: int, num_tokens: int = 1 << 30) -> bool:

@@ -372,3 +372,47 @@ def test_sgmv_errors_raise_runtime_error():
         sgmv.lora_a_sgmv_cutlass(x.float(), good_shrink, ptr, s, s, 0, 16)
     with pytest.raises(RuntimeError, match="int32"):
         sgmv.lora_a_sgmv_cutlass(x, good_shrink, ptr, s.long(), s.long(), 0, 16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("count,r,h_in,lens", [
+    (2, 64, 1024, [700, 1, 0, 33, 1, 300]),   # gate/up at rank 64: one launch of summed rank 128
+    (3, 16, 512, [520, 17, 64]),              # q/k/v at rank 16
+    (3, 40, 256, [1, 600, 5]),                # summed rank 120, not a multiple of 16 per projection
+    (4, 8, 384, [256, 257, 3]),               # four projections of rank 8
+    (4, 32, 1024, [900]),                     # summed rank 128
+    (3, 64, 512, [600, 40]),                  # summed rank 192: one launch per projection
+    (2, 16, 1000, [600, 40]),                 # h_in not a multiple of 128: one launch per projection
+    (2, 64, 1024, [100, 1, 30]),              # a small batch: the streaming kernel, one launch per projection
+])
+def test_sgmv_shrink_multi(dtype, count, r, h_in, lens):
+    """lorax_sgmv_shrink_multi: every projection's v as from lorax_sgmv_shrink on its own, whether the call
+    runs as one launch over the stacked A matrices or falls back to one launch per projection."""
+    print(f"case dtype={dtype} count={count} r={r} h_in={h_in} lens={lens}", flush=True)
+    gen = torch.Generator().manual_seed(count * 1000 + r + h_in)
+    starts, ends, pos = [], [], 2
+    for n in lens:
+        starts.append(pos)
+        ends.append(pos + n)
+        pos += n + 1  # one uncovered row after every segment
+    T, layer = pos, 1
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    stacks = [[randn((2, r, h_in), 0.05, gen, dtype, DEV) if n > 0 else None for n in lens] for _ in range(count)]
+    s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
+    tmp = sgmv.get_tmp_tensor(torch.device(DEV))
+    tables = [ptr_table(ws, DEV) for ws in stacks]
+    vs = sgmv.lora_a_sgmv_resident_multi(x, tmp, tables, s_start, s_end, layer, r)
+    singles = [sgmv.lora_a_sgmv_resident(x, tmp, t, s_start, s_end, layer, r) for t in tables]
+    torch.cuda.synchronize()
+    covered = torch.zeros(T, dtype=torch.bool)
+    for s, e in zip(starts, ends):
+        covered[s:e] = True
+    for p in range(count):
+        v_ref = torch.zeros((T, r), dtype=dtype)
+        for i, (s, e) in enumerate(zip(starts, ends)):
+            if e > s:
+                v_ref[s:e] = x.cpu()[s:e] @ stacks[p][i][layer].cpu().t()
+        assert_close(vs[p], v_ref, f"projection {p}")
+        assert_close(vs[p], singles[p].cpu(), f"projection {p} against its own launch")
+        assert torch.count_nonzero(vs[p].cpu()[~covered]) == 0
