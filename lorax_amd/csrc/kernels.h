@@ -96,16 +96,16 @@ struct SgmvArgs {
   size_t num_counters;
 };
 
-// Launch parameters that can be overridden from the environment for tuning runs
-// (LORAX_BGMV_LORA_BLOCKS, LORAX_BGMV_SHRINK_ROWS, LORAX_SHRINK_KSPLIT, LORAX_SHRINK_MB, LORAX_SHRINK_WAVES, LORAX_EXPAND_ROWS); 0 = heuristic.
+// Launch parameters that can be overridden from the environment for tuning runs, read once per process;
+// 0 (unset) = the launcher's heuristic.
 struct Tuning {
-  int bgmv_lora_blocks;
-  int bgmv_shrink_rows;
-  int shrink_ksplit;
-  int shrink_mb;
-  int shrink_waves;
-  int expand_rows;
-  int shrink_no_rotate;
+  int bgmv_lora_blocks;  // LORAX_BGMV_LORA_BLOCKS: expand blocks per workgroup of the single-launch BGMV (1, 2, 4)
+  int bgmv_shrink_rows;  // LORAX_BGMV_SHRINK_ROWS: rows of A per workgroup of the BGMV shrink (2, 4, 8)
+  int shrink_ksplit;     // LORAX_SHRINK_KSPLIT: K splits across workgroups of the register-operand SGMV shrink
+  int shrink_mb;         // LORAX_SHRINK_MB: 16-row blocks per row tile of the SGMV shrink (1, 2, 4)
+  int shrink_waves;      // LORAX_SHRINK_WAVES: waves per workgroup of the register-operand SGMV shrink
+  int expand_rows;       // LORAX_EXPAND_ROWS: rows per tile of the SGMV expand
+  int shrink_no_rotate;  // LORAX_SHRINK_NO_ROTATE: register-operand SGMV shrink without the K rotation per tile
   int shrink_lds;  // LORAX_SHRINK_LDS: 1 = always take the LDS-staged shrink where it applies, -1 = never
   int shrink_lds_kb;  // LORAX_SHRINK_LDS_KB: LDS budget of the staged shrink's buffers
   int bgmv_expand_cols;  // LORAX_BGMV_EXPAND_COLS: columns per lane group of the BGMV expand (4, 8, 16)
