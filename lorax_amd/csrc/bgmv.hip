@@ -279,22 +279,28 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
   }
 
   vec8 wv[U];
-  E yv[U][NT];
-  int col[U];
+  const int colbase = col0 + tid / CP;  // the lane group's column of step u is colbase + u * kCols
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    col[u] = col0 + u * kCols + tid / CP;
+    const int c = colbase + u * kCols;
     wv[u] = zero8<D>();
-    if (has_k && col[u] < h_out) wv[u] = load8<D>(B + static_cast<int64_t>(col[u]) * r + part * 8);
+    if (has_k && c < h_out) wv[u] = load8<D>(B + static_cast<int64_t>(c) * r + part * 8);
   }
+  // The y of step u belongs to lane u % CP of the column's lane group (after the shuffles every lane of
+  // the group holds the column's sum): a lane keeps ceil(U / CP) old values per token instead of U.
+  constexpr int UY = (U + CP - 1) / CP;
+  E yv[UY][NT];
 #pragma unroll
-  for (int u = 0; u < U; ++u)
+  for (int k = 0; k < UY; ++k) {
+    const int u = part + k * CP;
+    const int c = colbase + u * kCols;
 #pragma unroll
     for (int g = 0; g < NT; ++g) {
-      yv[u][g] = static_cast<E>(0.f);
-      if (part == 0 && col[u] < h_out && accumulate_into_y)
-        yv[u][g] = Y[static_cast<int64_t>(toks[g]) * y_stride + y_offset + col[u]];
+      yv[k][g] = static_cast<E>(0.f);
+      if (u < U && c < h_out && accumulate_into_y)
+        yv[k][g] = Y[static_cast<int64_t>(toks[g]) * y_stride + y_offset + c];
     }
+  }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     float s[NT];
@@ -304,11 +310,11 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
     for (int m = CP / 2; m >= 1; m >>= 1)
 #pragma unroll
       for (int g = 0; g < NT; ++g) s[g] += __shfl_xor(s[g], m, kWave);
-    if (part == 0 && col[u] < h_out) {
+    const int c = colbase + u * kCols;
+    if (part == u % CP && c < h_out) {
 #pragma unroll
       for (int g = 0; g < NT; ++g)
-        Y[static_cast<int64_t>(toks[g]) * y_stride + y_offset + col[u]] =
-            accumulate<D>(yv[u][g], s[g] * scale);
+        Y[static_cast<int64_t>(toks[g]) * y_stride + y_offset + c] = accumulate<D>(yv[u / CP][g], s[g] * scale);
     }
   }
 }
@@ -319,7 +325,7 @@ __device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const 
   using E = typename D::E;
   const int h_out = P.width;
   const int r = P.narrow;
-  const int col0 = slot.sub * (kBgmvThreads / CP) * U;
+  const int col0 = slot.sub * (kBgmvThreads / CP) * U;  // U = expand_steps(CP, the launch's U)
   int toks[kGroup];
   int64_t stack_addr;
   const int n = resolve_chunk(P, num_tokens, true, slot.chunk, toks, stack_addr);
@@ -341,6 +347,13 @@ __device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const 
       bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
       break;
   }
+}
+
+// Steps (columns per lane group) of an expand workgroup: ranks of 32 and more (4+ lanes per column) take
+// twice the launch's U - their lanes keep few old y values, so the registers allow it, and a wave then has
+// twice the bytes in flight.
+__host__ __device__ constexpr int expand_steps(int lanes_per_column, int u) {
+  return lanes_per_column >= 4 ? 2 * u : u;
 }
 
 // Lanes per column of a rank: the power of two >= r / 8.
@@ -365,13 +378,13 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBat
       bgmv_expand_problem<D, 2, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
     case 4:
-      bgmv_expand_problem<D, 4, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
+      bgmv_expand_problem<D, 4, expand_steps(4, U)>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
     case 8:
-      bgmv_expand_problem<D, 8, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
+      bgmv_expand_problem<D, 8, expand_steps(8, U)>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
     default:
-      bgmv_expand_problem<D, 16, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
+      bgmv_expand_problem<D, 16, expand_steps(16, U)>(P, vb, num_tokens, layer_idx, scale, acc_y);
       break;
   }
 }
@@ -741,7 +754,8 @@ static hipError_t launch_shrink(const BgmvArgs& a, hipStream_t stream) {
 template <typename D, int U>
 static hipError_t launch_expand_u(BgmvArgs a, hipStream_t stream) {
   const int64_t total = number_workgroups(a, [](const BgmvProblem& p) {
-    const int cols_per_wg = (kBgmvThreads / expand_lanes_per_column(p.narrow)) * U;
+    const int lanes = expand_lanes_per_column(p.narrow);
+    const int cols_per_wg = (kBgmvThreads / lanes) * expand_steps(lanes, U);
     return (p.width + cols_per_wg - 1) / cols_per_wg;
   });
   if (total == 0) return hipSuccess;
