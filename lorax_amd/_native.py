@@ -435,6 +435,9 @@ ESPACE = 5
 ENTRY_DTYPE = [("adapter", "<i8"), ("a_addr", "<i8"), ("b_addr", "<i8"), ("rank", "<i4"), ("reserved", "<i4")]
 
 
+_table_capacity = [64 * 1024, 64]  # bytes of packed tables, number of group records
+
+
 def build_batch_tables(adapter_indices, entries, entry_counts, prefill: bool):
     """lorax_build_batch_tables on numpy arrays: adapter_indices int64 [T]; entries a structured array of
     ENTRY_DTYPE, the layer types' adapters one after the other, each type sorted by adapter; entry_counts int32
@@ -448,18 +451,19 @@ def build_batch_tables(adapter_indices, entries, entry_counts, prefill: bool):
     bounds = np.zeros(T + 1, dtype=np.int32)
     owners = np.zeros(max(T, 1), dtype=np.int64)
     nseg, ngroups, nbytes = _c.c_int32(0), _c.c_int32(0), _c.c_int64(0)
-    capacity, group_capacity = 64 * 1024, 64
+    capacity, group_capacity = _table_capacity
     while True:
-        packed = np.zeros(capacity, dtype=np.uint8)
+        packed = np.empty(capacity, dtype=np.uint8)  # the builder writes every byte it reports as used
         groups = (TableGroup * group_capacity)()
         rc = lib().lorax_build_batch_tables(
             adapter_indices.ctypes.data, T, entries.ctypes.data, entry_counts.ctypes.data, entry_counts.shape[0],
             1 if prefill else 0, bounds.ctypes.data, owners.ctypes.data, ctypes.byref(nseg), packed.ctypes.data,
             capacity, ctypes.byref(nbytes), groups, group_capacity, ctypes.byref(ngroups),
         )
-        if rc == ESPACE:
-            capacity = max(capacity, int(nbytes.value))
-            group_capacity = max(group_capacity, int(ngroups.value))
+        if rc == ESPACE:  # remembered: the next batch of this size takes one call
+            capacity = max(capacity, int(nbytes.value) * 5 // 4)
+            group_capacity = max(group_capacity, int(ngroups.value) * 2)
+            _table_capacity[:] = [capacity, group_capacity]
             continue
         if rc != 0:
             _raise_last(rc)

@@ -421,14 +421,23 @@ class LayerAdapterWeights:
     def __init__(self):
         self.adapter_weights: Dict[int, AdapterWeights] = {}
         self._lora_entries = None  # cached argument of the native table builder
+        self._unwrapped = None
 
     def add_adapter(self, adapter_idx: int, weights: AdapterWeights):
         self.adapter_weights[adapter_idx] = weights
         self._lora_entries = None
+        self._unwrapped = None
 
     def remove_adapter(self, adapter_idx: int):
         self.adapter_weights.pop(adapter_idx, None)
         self._lora_entries = None
+        self._unwrapped = None
+
+    def unwrapped(self) -> Dict[int, "AdapterWeights"]:
+        """adapter index -> the adapter's weights without their wrapper; rebuilt only when adapters come or go."""
+        if self._unwrapped is None:
+            self._unwrapped = {idx: _unwrap(w) for idx, w in self.adapter_weights.items()}
+        return self._unwrapped
 
     def lora_entries(self):
         """(adapter, address of the [L, r, h_in] stack, address of the [L, h_out, r] stack, rank) of every LoRA
@@ -594,6 +603,7 @@ def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAda
     dev = torch.from_numpy(packed).to(device)
     dev64, dev32 = dev.view(torch.int64), dev.view(torch.int32)
     seg_adapters = owners.tolist()
+    batch_adapters = set(seg_adapters)
     T = int(indices.shape[0])
 
     by_type: Dict[int, List] = defaultdict(list)
@@ -603,7 +613,8 @@ def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAda
     for lt, type_groups in by_type.items():
         layer_name = names[lt]
         layer = weights[layer_name]
-        loras = {a: _unwrap(layer.adapter_weights[a]) for a in set(seg_adapters) if a in layer.adapter_weights}
+        every = layer.unwrapped()
+        loras = {a: every[a] for a in batch_adapters if a in every}
         use_sgmv = bool(type_groups[0].use_sgmv)
         null = EMPTY_TENSOR.data_ptr()
 
@@ -618,12 +629,18 @@ def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAda
             b_ptr = dev64[g.b_ptr_off // 8 : g.b_ptr_off // 8 + n]
             if use_sgmv:
                 tmp_shrink, tmp_expand = get_tmp_tensors(n, g.rank, device)
-                segs = [s for s, a in enumerate(seg_adapters) if a in loras and loras[a].lora_a_r == g.rank]
-                segs.sort(key=_segment_order(segs, seg_adapters, bounds.tolist()))
+
+                def ref_table(layout: str, rank=g.rank, loras=loras, table=table) -> torch.Tensor:
+                    # the group's segments in the builder's order (only computed if somebody asks for the
+                    # reference-layout tables)
+                    segs = [s for s, a in enumerate(seg_adapters) if a in loras and loras[a].lora_a_r == rank]
+                    segs.sort(key=_segment_order(segs, seg_adapters, bounds.tolist()))
+                    return table(layout)[segs]
+
                 rank_data[g.rank] = RankSegments(
                     rank=g.rank,
-                    lora_a_ptr=(lambda segs=segs, table=table: table("weights_a")[segs]),
-                    lora_b_ptr=(lambda segs=segs, table=table: table("weights_b")[segs]),
+                    lora_a_ptr=(lambda ref_table=ref_table: ref_table("weights_a")),
+                    lora_b_ptr=(lambda ref_table=ref_table: ref_table("weights_b")),
                     tmp_shrink=tmp_shrink,
                     tmp_expand=tmp_expand,
                     segment_starts=dev32[g.starts_off // 4 : g.starts_off // 4 + n],

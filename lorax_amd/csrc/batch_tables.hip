@@ -21,11 +21,12 @@ struct Packer {
   char* base;
   int64_t capacity;
   int64_t used = 0;
-  // Reserves `bytes` (16-byte aligned); returns the offset.  Keeps counting past the capacity so that the
-  // caller learns the size it needs.
+  // Reserves `bytes` (16-byte aligned, the padding zeroed); returns the offset.  Keeps counting past the
+  // capacity so that the caller learns the size it needs.
   int64_t reserve(int64_t bytes) {
     const int64_t off = used;
     used += (bytes + 15) / 16 * 16;
+    if (used <= capacity && used > off + bytes) std::memset(base + off + bytes, 0, used - off - bytes);
     return off;
   }
   template <typename T>
@@ -72,6 +73,8 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
   std::vector<std::vector<int32_t>> group_segs;  // segments of each rank group
   std::vector<int32_t> slot_of_seg(num_segments);
   std::vector<int32_t> token_seg(num_tokens);
+  std::vector<int32_t> slot_count, slot_begin, slot_fill, slot_order, toks_by_slot(num_tokens), entry_first;
+  std::vector<int64_t> entry_rows;
   for (int32_t s = 0; s < num_segments; ++s)
     for (int32_t t = segment_bounds[s]; t < segment_bounds[s + 1]; ++t) token_seg[t] = s;
 
@@ -88,6 +91,7 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
         max_rank = std::max(max_rank, static_cast<int>(seg_entry[s]->rank));
       }
     }
+    const lorax_adapter_entry_t* type_first = type_entries;
     type_entries += count;
     if (!any) continue;
     const bool use_sgmv = prefill != 0 || max_rank > kBgmvMaxRank;  // lora.py:311
@@ -115,13 +119,11 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
       // several of them would otherwise be streamed once per token.  Adapters with the most rows come first,
       // so that the long tiles of a launch start early.  Stable: (rows of the adapter, descending; adapter).
       if (use_sgmv) {
+        // rows per adapter, indexed by the adapter's position in this layer type's entry list
+        entry_rows.assign(count, 0);
+        for (int32_t x : segs) entry_rows[seg_entry[x] - type_first] += segment_bounds[x + 1] - segment_bounds[x];
         std::vector<int64_t> rows_of(num_segments, 0);
-        for (int32_t x : segs) {
-          int64_t rows = 0;
-          for (int32_t y : segs)
-            if (segment_owners[y] == segment_owners[x]) rows += segment_bounds[y + 1] - segment_bounds[y];
-          rows_of[x] = rows;
-        }
+        for (int32_t x : segs) rows_of[x] = entry_rows[seg_entry[x] - type_first];
         std::stable_sort(segs.begin(), segs.end(), [&](int32_t x, int32_t y) {
           if (rows_of[x] != rows_of[y]) return rows_of[x] > rows_of[y];
           return segment_owners[x] < segment_owners[y];
@@ -156,35 +158,43 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
         // slot of a token = position of the FIRST segment of its adapter inside this group's pointer slice
         // (lora.py:354-366); tokens of other ranks, of adapters without weights here and of no adapter: -1.
         std::fill(slot_of_seg.begin(), slot_of_seg.end(), -1);
+        entry_first.assign(count, -1);  // first position of an adapter in the group, by entry position
         for (int32_t i = 0; i < n; ++i) {
-          int32_t first = i;
-          for (int32_t j = 0; j < i; ++j)
-            if (segment_owners[segs[j]] == segment_owners[segs[i]]) { first = j; break; }
+          int32_t& first = entry_first[seg_entry[segs[i]] - type_first];
+          if (first < 0) first = i;
           slot_of_seg[segs[i]] = first;
         }
         desc.indices_off = pack.reserve(num_tokens * 8);
         int64_t* idx = pack.at<int64_t>(desc.indices_off);
         // chunks: tokens of one slot, in token order, cut into groups of kPlanGroup; slots in order of their
-        // first token
-        std::vector<std::vector<int32_t>> toks_of_slot(n);
-        std::vector<int32_t> slot_order;
+        // first token.  Counting sort of the tokens by slot (flat arrays, no allocation per slot).
+        slot_count.assign(n, 0);
+        slot_order.clear();
         for (int64_t t = 0; t < num_tokens; ++t) {
           const int32_t slot = slot_of_seg[token_seg[t]];
           if (idx != nullptr) idx[t] = slot;
-          if (slot >= 0) {
-            if (toks_of_slot[slot].empty()) slot_order.push_back(slot);
-            toks_of_slot[slot].push_back(static_cast<int32_t>(t));
-          }
+          if (slot >= 0 && slot_count[slot]++ == 0) slot_order.push_back(slot);
         }
-        int32_t chunks = 0;
-        for (int32_t slot : slot_order) chunks += (static_cast<int32_t>(toks_of_slot[slot].size()) + kPlanGroup - 1) / kPlanGroup;
+        slot_begin.assign(n, 0);
+        int32_t chunks = 0, placed = 0;
+        for (int32_t slot : slot_order) {
+          slot_begin[slot] = placed;
+          placed += slot_count[slot];
+          chunks += (slot_count[slot] + kPlanGroup - 1) / kPlanGroup;
+        }
         desc.num_chunks = chunks;
         desc.plan_off = pack.reserve(static_cast<int64_t>(chunks) * lorax::kPlanRecordWords * 8);
         if (int64_t* rec = pack.at<int64_t>(desc.plan_off)) {
+          slot_fill = slot_begin;
+          for (int64_t t = 0; t < num_tokens; ++t) {
+            const int32_t slot = slot_of_seg[token_seg[t]];
+            if (slot >= 0) toks_by_slot[slot_fill[slot]++] = static_cast<int32_t>(t);
+          }
           for (int32_t slot : slot_order) {
-            const std::vector<int32_t>& toks = toks_of_slot[slot];
-            for (size_t i = 0; i < toks.size(); i += kPlanGroup) {
-              const int cnt = static_cast<int>(std::min<size_t>(kPlanGroup, toks.size() - i));
+            const int32_t* toks = toks_by_slot.data() + slot_begin[slot];
+            const int32_t total = slot_count[slot];
+            for (int32_t i = 0; i < total; i += kPlanGroup) {
+              const int cnt = std::min<int32_t>(kPlanGroup, total - i);
               rec[0] = cnt;
               for (int q = 0; q < kPlanGroup; ++q) rec[1 + q] = toks[q < cnt ? i + q : i];
               rec[5] = seg_entry[segs[slot]]->a_addr;
