@@ -3,9 +3,11 @@
 //
 // Same arithmetic and rounding as sgmv_expand.hip.  The MFMA product is v (16 rows of a block, first
 // operand) times B (second operand), and with B^T in memory the second operand needs no transposition:
-// lane (c, g) of accumulator j reads the 16 bytes B^T[column(j, c)][32 s + 8 g ...] straight from global
-// memory.  There is no LDS staging, no barrier and no LDS gather in a tile's prologue - which, for the
-// short segments a prefill batch is full of, took longer than the rows themselves.
+// the 16 bytes B^T[column(j, c)][32 s + 8 g ...] that lane (c, g) of accumulator j needs come straight from
+// global memory into registers (fetched by the lane that makes the access contiguous and handed over with
+// a cross-lane move, see the kernel).  There is no LDS staging, no barrier and no LDS gather in a tile's
+// prologue - which, for the short segments a prefill batch is full of, took longer than the rows
+// themselves.
 //
 // The columns of a wave's panel are dealt to the accumulators so that a lane ends up with NJ ADJACENT
 // columns of four rows (see the kernel).  A y access of the wave is then four whole runs of 32 * NJ
@@ -55,12 +57,27 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
   const int panel0 = (vid / tile_slots) * kExpTWaves * panels_per_wave;
   const bool acc_y = accumulate_into_y != 0;
 
-  bool k_ok[KS];
-  int k_off[KS];
+  // MFMA operand layout: lane g * 16 + c holds the eight k values 32 s + 8 g ... of operand row / column c.
+  // Fetched that way, neighbouring lanes read different rows, r * 2 bytes apart, and every 16-byte piece
+  // is a cache-line lookup of its own.  So the operands are FETCHED with lane l taking piece l & 3 of row
+  // l >> 2 - a quad of lanes reads 64 contiguous bytes - and then change lanes through the LDS crossbar
+  // (ds_bpermute, no LDS memory): the lane g * 16 + c takes the registers of lane 4 c + g.
+  const int lc = lane >> 2;
+  const int from_lane = (c * 4 + g) * 4;  // ds_bpermute addresses lanes in bytes
+  auto to_operand_lanes = [&](vec8 fetched) {
+    const u32x4 raw = __builtin_bit_cast(u32x4, fetched);
+    u32x4 mine;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+      mine[d] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(from_lane, static_cast<int>(raw[d])));
+    return __builtin_bit_cast(vec8, mine);
+  };
+  bool k_ok[KS];  // of the operand lane: chunks beyond the rank are zeroed after the exchange
+  int l_off[KS];  // of the fetching lane: chunks beyond the rank are fetched from chunk 0
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
-    k_ok[s] = s * 32 + g * 8 < r;  // chunks beyond the rank are loaded from chunk 0 and zeroed
-    k_off[s] = k_ok[s] ? s * 32 + g * 8 : 0;
+    k_ok[s] = s * 32 + g * 8 < r;
+    l_off[s] = s * 32 + (lane & 3) * 8 < r ? s * 32 + (lane & 3) * 8 : 0;
   }
 
   for (int tile = vid % tile_slots;; tile += tile_slots) {
@@ -86,9 +103,11 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
       const uint32_t ystride = static_cast<uint32_t>(y_stride);
       const int last = rt.row_end - rt.row0 - 1;
       auto load_block = [&](int mb, vec8(&vf)[KS], yvec(&yv)[4]) {
-        const uint32_t voff = static_cast<uint32_t>(min(mb * 16 + c, last)) * static_cast<uint32_t>(r);
+        // v rows are fetched like the B^T rows below: lane l takes piece l & 3 of row l >> 2 of the block, and
+        // finish_block moves the pieces to the lanes the MFMA wants them in
+        const uint32_t voff = static_cast<uint32_t>(min(mb * 16 + lc, last)) * static_cast<uint32_t>(r);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) vf[s] = load8<D>(vtile + (voff + k_off[s]));
+        for (int s = 0; s < KS; ++s) vf[s] = load8<D>(vtile + (voff + l_off[s]));
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t row = static_cast<uint32_t>(min(mb * 16 + g * 4 + i, last));
@@ -102,16 +121,20 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
       yvec yr[kExpTStages][4];
 #pragma unroll
       for (int s = 0; s < kExpTStages - 1; ++s) load_block(block_of(s), vr[s], yr[s]);
+      // B^T operands: lane l fetches piece l & 3 of the row of operand column l >> 2
       vec8 bf[NJ][KS];
+      const int lcol = (n0 + NJ * lc < h_out) ? n0 + NJ * lc : n0;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
 #pragma unroll
         for (int s = 0; s < KS; ++s)
-          bf[j][s] = keep_if<D>(k_ok[s], load8<D>(BT + static_cast<int64_t>(col + j) * r + k_off[s]));
+          bf[j][s] = keep_if<D>(k_ok[s], to_operand_lanes(load8<D>(BT + static_cast<int64_t>(lcol + j) * r + l_off[s])));
       }
 
       auto finish_block = [&](bool live, int mb, vec8(&vf)[KS], yvec(&yv)[4]) {
         f32x4 acc[NJ];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) vf[s] = to_operand_lanes(vf[s]);
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
           acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
