@@ -1,6 +1,7 @@
 """The six LoRA operators of lorax_server/utils/ops (bgmv_shrink / bgmv_expand / bgmv_expand_slice /
-sgmv_shrink / sgmv_expand / sgmv_expand_slice) on the HIP kernels of this package, plus bgmv_lora_slices,
-which runs the decode update of several column slices in two launches.
+sgmv_shrink / sgmv_expand / sgmv_expand_slice) on the HIP kernels of this package, plus bgmv_lora_slices
+and sgmv_lora_slices, which run the update of several column slices that share their input with one shrink
+launch for all of them (decode: and one expand launch).
 
 Same names, argument orders and meaning as the reference's Triton operators, which index ONE stacked
 weight tensor per layer - lora_a_weights [num_loras, r, h_in], lora_b_weights [num_loras, h_out, r], an
@@ -223,6 +224,52 @@ def sgmv_shrink(
                         get_tmp_tensor(inputs.device), 0, scaling)
     if finish is not None:
         finish()
+
+
+@torch.inference_mode()
+def sgmv_lora_slices(
+    inputs: torch.Tensor,
+    slices,
+    output_tensor: torch.Tensor,
+    b_seq_start_loc: torch.Tensor,
+    seq_len_tensor: torch.Tensor,
+    lora_indices_tensor: torch.Tensor,
+    batches: int,
+    max_seq_length: int,
+    scaling: float = 1.0,
+    bounds: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+):
+    """sgmv_shrink followed by sgmv_expand_slice(add_inputs=True) for several column slices of output_tensor that
+    share `inputs` (q/k/v, gate/up): `slices` is a sequence of (lora_a_weights, lora_b_weights, slice_offset,
+    slice_size).  No counterpart among the reference's operators (its wrapper calls them once per slice,
+    punica.py:750-773): slices of one rank shrink together, up to a summed rank of 128 per launch, so `inputs`
+    is read once per launch; the intermediate is kept in the type of `inputs`."""
+    assert inputs.dtype in (torch.float16, torch.bfloat16)
+    assert inputs.is_contiguous() and output_tensor.is_contiguous()
+    assert inputs.size(0) == output_tensor.size(0)
+    assert b_seq_start_loc.size(0) == batches and lora_indices_tensor.size(0) == batches
+    s_start, s_end = bounds if bounds is not None else segment_bounds(b_seq_start_loc, seq_len_tensor,
+                                                                        lora_indices_tensor)
+    by_rank: Dict[int, list] = {}
+    for lora_a_weights, lora_b_weights, slice_offset, slice_size in slices:
+        a = _stacked(lora_a_weights, "lora_a_weights")
+        b = _stacked(lora_b_weights, "lora_b_weights")
+        assert a.dtype == inputs.dtype and b.dtype == inputs.dtype
+        assert inputs.size(1) == a.size(-1) and a.size(-2) == b.size(-1) and slice_size == b.size(-2)
+        by_rank.setdefault(a.size(-2), []).append((a, b, slice_offset, slice_size))
+    tmp = get_tmp_tensor(inputs.device)
+    tmp_expand = get_tmp_tensor_for_size(batches, inputs.device)
+    tokens = inputs.size(0)
+    for r, jobs in by_rank.items():
+        step = max(1, min(_native.MAX_SGMV_SHRINK_PROBLEMS, 128 // r))
+        for i in range(0, len(jobs), step):
+            chunk = jobs[i : i + step]
+            bufs = list(torch.zeros((len(chunk), tokens, r), dtype=inputs.dtype, device=inputs.device).unbind(0))
+            _native.sgmv_shrink_multi(bufs, inputs, [_segment_pointers(a, lora_indices_tensor) for a, _, _, _ in chunk],
+                                      s_start, s_end, tmp, 0, scaling)
+            for v, (_, b, off, size) in zip(bufs, chunk):
+                _native.sgmv_expand(output_tensor, v, _segment_pointers(b, lora_indices_tensor), s_start, s_end,
+                                    tmp_expand, 0, off, size, transposed=True, accumulate=True)
 
 
 @torch.inference_mode()

@@ -195,16 +195,21 @@ class PunicaWrapper:
     def add_lora_slices(self, y: torch.Tensor, x: torch.Tensor, slices, scale: float,
                         callback: Optional[Callable] = None) -> None:
         """add_lora for several column slices of y that share x; `slices` is a sequence of
-        (wa_t_all, wb_t_all, y_offset, y_slice_size).  In decode, without a callback between shrink and expand,
-        all shrinks are one launch and all expands another; otherwise one add_lora per slice."""
+        (wa_t_all, wb_t_all, y_offset, y_slice_size).  Without a callback between shrink and expand the shrinks
+        of the slices run together (decode: one launch, and one for all expands; prefill: one launch per summed
+        rank of 128); otherwise one add_lora per slice."""
         if not slices:
             return
         y2 = y.view(-1, y.shape[-1])
         x2 = x.view(-1, x.shape[-1])
-        batched = (not self.is_prefill and callback is None and x2.dtype in (torch.float16, torch.bfloat16)
+        batched = (callback is None and x2.dtype in (torch.float16, torch.bfloat16)
                    and all(wa.dtype == x2.dtype and wb.dtype == x2.dtype for wa, wb, _, _ in slices))
-        if batched:
+        if batched and not self.is_prefill:
             ops.bgmv_lora_slices(x2, slices, y2, self.token_lora_indices, scale)
+            return
+        if batched:
+            if not self.no_lora:  # punica.py:557-559
+                ops.sgmv_lora_slices(x2, slices, y2, *self.prefill_metadata, scale, bounds=self._bounds)
             return
         for wa_t_all, wb_t_all, y_offset, y_slice_size in slices:
             whole = y_offset == 0 and y_slice_size == y2.shape[1]

@@ -158,18 +158,20 @@ def test_add_lora_through_the_layer_matches_the_pointer_table_path(prefill):
 
 @pytest.mark.parametrize("prefill", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_add_lora_packed_nslice(prefill, dtype):
-    """PunicaWrapper.add_lora_packed_nslice (punica.py:750-773) over three slices of different rank: in decode
-    the shrinks are one launch and the expands another; the result is add_lora slice by slice."""
-    print(f"case prefill={prefill} dtype={dtype}", flush=True)
+@pytest.mark.parametrize("ranks,repeat", [((8, 16, 64), 1), ((16, 16, 16), 1), ((32, 32, 32), 16)])
+def test_add_lora_packed_nslice(prefill, dtype, ranks, repeat):
+    """PunicaWrapper.add_lora_packed_nslice (punica.py:750-773) over three slices: in decode the shrinks are one
+    launch and the expands another; in prefill slices of one rank shrink together (one launch over the stacked
+    A matrices once the batch has more than 512 rows); the result is add_lora slice by slice."""
+    print(f"case prefill={prefill} dtype={dtype} ranks={ranks} repeat={repeat}", flush=True)
     gen = torch.Generator().manual_seed(17)
-    h_in, sizes, ranks, n = 1024, (1024, 264, 256), (8, 16, 64), 4
-    token_idx = [-1] * 2 + [0] * 9 + [2] * 1 + [-1] * 1 + [1] * 20 + [2] * 3 + [3] * 5
+    h_in, sizes, n = 1024, (1024, 264, 256), 4
+    token_idx = ([-1] * 2 + [0] * 9 + [2] * 1 + [-1] * 1 + [1] * 20 + [2] * 3 + [3] * 5) * repeat
     T = len(token_idx)
     stacks = [_stacks(n, r, h_in, h_out, gen, dtype) for r, h_out in zip(ranks, sizes)]
     x = randn((T, h_in), 1.0, gen, dtype, DEV)
     y0 = randn((T, sum(sizes)), 0.5, gen, dtype, DEV)
-    wrapper = PunicaWrapper(max_num_batched_tokens=64, max_batches=64, device=DEV, enabled=True)
+    wrapper = PunicaWrapper(max_num_batched_tokens=1024, max_batches=256, device=DEV, enabled=True)
     # token_adapters of the batch: adapter index i + 1 is stack entry i, index 0 is the base model
     wrapper.update_metadata(make_meta([i + 1 for i in token_idx], torch.device(DEV)), prefill)
     assert wrapper.token_lora_indices.tolist() == token_idx
@@ -186,6 +188,9 @@ def test_add_lora_packed_nslice(prefill, dtype):
         y_ref = _ref_lora(y_ref, x.cpu(), a, b, token_idx, 0.5, off, size, dtype)
         off += size
     assert_close(y, y_ref, "add_lora_packed_nslice", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
-    assert torch.equal(y.cpu(), y_each.cpu())  # same kernels, same arithmetic, one launch or three
+    if prefill:  # the grouped shrink sums in another order than a projection's own launch
+        assert_close(y, y_each.cpu(), "grouped against slice by slice", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
+    else:
+        assert torch.equal(y.cpu(), y_each.cpu())  # same kernels, same arithmetic, one launch or three
     routed = torch.tensor(token_idx) >= 0
     assert torch.equal(y.cpu()[~routed], y0.cpu()[~routed])
