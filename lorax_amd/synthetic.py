@@ -51,7 +51,11 @@ class Workload:
     inputs: Dict[str, torch.Tensor] = field(default_factory=dict)  # group name -> [T, h_in]
     weights: Dict[str, LayerAdapterWeights] = field(default_factory=dict)  # layer name -> adapters
     meta: Optional[AdapterBatchMetadata] = None
-    extra_segments: List[Tuple[int, int, int]] = field(default_factory=list)  # (start, end, adapter)
+    # Segments added to every rank group's tables after they are built: (start, end, adapter) with
+    # end <= start, adapter None = a null stack address.  A serving loop produces such entries when it
+    # pads its tables to a fixed size (the reference's own SGMV test passes them, server/tests/utils/
+    # test_sgmv.py:46-47); the run-length routing of a real batch never does.
+    extra_segments: List[Tuple[int, int, Optional[int]]] = field(default_factory=list)
 
     @property
     def num_tokens(self) -> int:
@@ -64,7 +68,59 @@ class Workload:
         return len({a for a in self.adapter_indices if a in self.rank_of_adapter})
 
     def batch_data(self) -> AdapterBatchData:
-        return AdapterBatchData.from_meta(self.meta, self.weights, {}, None, self.prefill, None)
+        batch = AdapterBatchData.from_meta(self.meta, self.weights, {}, None, self.prefill, None)
+        if self.extra_segments and self.prefill:
+            _inject_segments(self, batch)
+        return batch
+
+
+def _splice_rank_group(rs, layer, rank: int, extra) -> None:
+    """Adds the segments `extra` to one rank group's tables: the first one in front of the group's second
+    segment, the others at the end."""
+    from lorax_amd.sgmv import get_tmp_tensors
+
+    n = rs.segment_starts.numel()
+    at = [min(1, n)] + [n] * (len(extra) - 1)  # insertion points in the original table
+
+    def spliced(table, values, dtype):
+        parts, prev = [], 0
+        for pos, val in zip(at, values):
+            parts += [table[prev:pos], torch.tensor([val], dtype=dtype, device=table.device)]
+            prev = pos
+        parts.append(table[prev:])
+        return torch.cat(parts)
+
+    def addrs(layout):
+        out = []
+        for _, _, adapter in extra:
+            lw = layer.get(adapter) if adapter is not None else None
+            out.append(getattr(lw, layout).data_ptr() if lw is not None and lw.lora_a_r == rank else 0)
+        return out
+
+    def later(old, layout):  # the reference-layout tables are built on first access
+        return lambda: spliced(old() if callable(old) else old, addrs(layout), torch.int64)
+
+    rs._lora_a_ptr = later(rs._lora_a_ptr, "weights_a")
+    rs._lora_b_ptr = later(rs._lora_b_ptr, "weights_b")
+    rs.lora_a_t_ptr = spliced(rs.lora_a_t_ptr, addrs("weights_a_t"), torch.int64)
+    rs.lora_b_t_ptr = spliced(rs.lora_b_t_ptr, addrs("weights_b_t"), torch.int64)
+    rs.segment_starts = spliced(rs.segment_starts, [s for s, _, _ in extra], torch.int32)
+    rs.segment_ends = spliced(rs.segment_ends, [e for _, e, _ in extra], torch.int32)
+    rs.tmp_shrink, rs.tmp_expand = get_tmp_tensors(n + len(extra), rank, rs.segment_starts.device)
+    if rs.segments_key is not None:
+        rs.segments_key = (rs.segments_key, tuple(extra))
+
+
+def _inject_segments(w: "Workload", batch: AdapterBatchData) -> None:
+    """Adds w.extra_segments to the segment tables of every rank group of a prefill batch."""
+    from lorax_amd.adapters import LORA
+
+    for name, per_type in batch.data.items():
+        data = per_type.get(LORA)
+        if data is None or not data.use_sgmv:
+            continue
+        for rank, rs in data.rank_data.items():
+            _splice_rank_group(rs, w.weights[name].adapter_weights, rank, w.extra_segments)
 
 
 def _randn(shape, std, gen, dtype, device):
@@ -187,11 +243,13 @@ def config4(device, num_layers: int = 2, weights_on_device: bool = True, num_tok
 
 def config5(device, num_layers: int = 1, weights_on_device: bool = True, prefill_tokens: int = 4096,
             decode_tokens: int = 256, num_adapters: int = 256, groups: Optional[List[ProjectionGroup]] = None,
-            resident_only_active: bool = True) -> Workload:
+            resident_only_active: bool = False) -> Workload:
     """bf16 mixed batch on a Llama-70B-shaped layer: one chunked-prefill run plus single-token decode runs,
-    rank-128 adapters, a run of tokens whose adapter has no weights, and tokens with no adapter at all.
-    The whole batch is routed by segments, as the reference does for any batch with a prefilling request
-    (flash_causal_lm.py:1594,1617)."""
+    `num_adapters` resident rank-128 adapters, a run of tokens whose adapter has no weights, tokens with no
+    adapter at all, and two empty entries in every rank group's segment tables: one with start == end and a
+    valid stack address, one (-1, -1) with a null address.  The whole batch is routed by segments, as the
+    reference does for any batch with a prefilling request (flash_causal_lm.py:1594,1617).
+    resident_only_active keeps weights only for the adapters the batch uses (for tests on small memory)."""
     gen = torch.Generator(device="cpu").manual_seed(1005)
     dec = torch.randint(0, num_adapters, (decode_tokens,), generator=gen).tolist()
     no_weights_adapter = num_adapters  # resident nowhere: its runs are dropped from every rank group
@@ -206,7 +264,17 @@ def config5(device, num_layers: int = 1, weights_on_device: bool = True, prefill
         rank_of = {a: r for a, r in rank_of.items() if a in active}
     w = Workload("cfg5_llama70b_mixed_prefill_decode", torch.bfloat16, torch.device(device), num_layers, True,
                  groups if groups is not None else LLAMA70B_LAYER, idx, rank_of)
+    w.extra_segments = [(prefill_tokens // 2, prefill_tokens // 2, dec[0]), (-1, -1, None)]
     _populate(w, 1005, weights_on_device)
+    return w
+
+
+def mid_prefill(device, num_layers: int = 16, weights_on_device: bool = True, num_segments: int = 10) -> Workload:
+    """bf16 prefill of about a thousand tokens (10 runs of 32..256 tokens, one rank-64 adapter each) on the
+    Mistral-7B MLP: the band between the streaming shrink (a few hundred rows) and batches with enough row tiles
+    for every CU; not one of the five benchmark configurations."""
+    w = config3(device, num_layers, weights_on_device, num_segments=num_segments, min_len=32, max_len=256)
+    w.name = "mid_prefill_1k_mlp"
     return w
 
 

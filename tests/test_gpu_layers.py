@@ -73,6 +73,21 @@ def _check_workload(w, layer_id, y0_std):
         assert torch.equal(out.cpu()[untouched], y0[untouched]), "rows without an adapter must be bit-identical"
 
 
+def assert_has_empty_segments(w, batch):
+    """Every rank group of a cfg5 batch carries an empty segment with a valid stack address (start == end) and
+    a (-1, -1) segment with a null address, next to its real segments."""
+    seen = 0
+    for per_type in batch.data.values():
+        for rd in per_type[LORA].rank_data.values():
+            rows = list(zip(rd.segment_starts.tolist(), rd.segment_ends.tolist(), rd.lora_a_t_ptr.tolist(),
+                            rd.lora_b_t_ptr.tolist()))
+            assert any(s == e and s >= 0 and a != 0 and b != 0 for s, e, a, b in rows), rows
+            assert any(s == -1 and e == -1 and a == 0 and b == 0 for s, e, a, b in rows), rows
+            assert rd.tmp_expand.numel() == 60 * len(rows)
+            seen += 1
+    assert seen > 0
+
+
 def test_config1_llama7b_q_proj_prefill():
     w = synthetic.config1(DEV, num_layers=2)
     assert w.meta.adapter_segments.tolist() == [0, 16, 32, 48, 64] and w.meta.segment_indices == [0, 1, 2, 3]
@@ -120,8 +135,11 @@ def test_config5_llama70b_mixed_batch_reduced():
     rd = data.rank_data[128]
     lens = (rd.segment_ends - rd.segment_starts).tolist()
     assert max(lens) >= 300 and lens.count(1) >= 10
-    # the run whose adapter has no weights and the run with no adapter are in no rank group
-    assert len(lens) < len(w.meta.segment_indices)
+    # the run whose adapter has no weights and the run with no adapter are in no rank group; two empty
+    # entries were added to the tables
+    assert len(lens) - 2 < len(w.meta.segment_indices)
+    assert_has_empty_segments(w, batch)
+    assert len(w.rank_of_adapter) == 16  # every adapter resident, not only the batch's
     _check_workload(w, 0, 0.25)
 
 
@@ -129,4 +147,5 @@ def test_config5_mlp_projections_reduced():
     groups = [g for g in synthetic.LLAMA70B_LAYER if g.name in ("gate_up", "down_proj")]
     w = synthetic.config5(DEV, num_layers=1, weights_on_device=False, prefill_tokens=130, decode_tokens=8,
                           num_adapters=6, groups=groups)
+    assert_has_empty_segments(w, w.batch_data())
     _check_workload(w, 0, 0.25)

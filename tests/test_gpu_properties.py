@@ -12,7 +12,7 @@ from lorax_amd.adapters import AdapterBatchData
 from lorax_amd.synthetic import make_meta
 from oracle import lora_oracle as O
 from tests.helpers import assert_close, ptr_table
-from tests.test_gpu_layers import _run_group
+from tests.test_gpu_layers import _run_group, assert_has_empty_segments
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -72,7 +72,10 @@ def test_cfg4_full_size_sampled_rows():
 
 
 def test_cfg5_full_size_sampled_rows():
-    _check_sampled(synthetic.config5(DEV, num_layers=1, weights_on_device=True), 0, sample=64)
+    w = synthetic.config5(DEV, num_layers=1, weights_on_device=True)
+    assert len(w.rank_of_adapter) == 256 and w.distinct_adapters() < 256  # all 256 adapters are resident
+    assert_has_empty_segments(w, w.batch_data())
+    _check_sampled(w, 0, sample=64)
 
 
 @pytest.mark.parametrize("config", [2, 4])
