@@ -6,8 +6,8 @@
  * `punica_kernels` (server/punica_kernels/punica_kernels/punica_ops.cc:446-459).
  * All pointers are device pointers in the current HIP device's memory unless the
  * comment says otherwise.  `stream` is a hipStream_t passed as void* (NULL = the
- * default stream).  No entry point allocates, frees or synchronises; every one is
- * safe to call while `stream` is being captured into a HIP graph.
+ * default stream).  No entry point allocates, frees or synchronises, and none keeps state
+ * between calls; every one is safe to call while `stream` is being captured into a HIP graph.
  *
  * Return value: 0 on success, a LORAX_E* code otherwise; the message for the last
  * failure on the calling thread is returned by lorax_last_error().  Errors are
@@ -156,9 +156,14 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
  *   legacy path; the `scaling` argument of lorax_server/utils/ops/sgmv_shrink.py:101-196).
  *
  * r must be a multiple of 8 in [8, 128]; h_in a multiple of 8; LORAX_A_RH with a rank that is not a
- * multiple of 16 additionally needs h_in to be a multiple of 128 or num_tokens <= 512.  `tmp`/`tmp_bytes` is the caller's
- * scratch and is only validated for presence; the split-K partial sums live in the
- * library's own per-device workspace (see lorax_init).
+ * multiple of 16 additionally needs h_in to be a multiple of 128 or num_tokens <= 512.
+ *
+ * `tmp`/`tmp_bytes` is the caller's scratch, with the reference's sizes (8 MiB for LORAX_A_RH, punica_ops.cc:
+ * 389-390; lorax_sgmv_tmp_size(num_segments) for LORAX_A_HR, punica_ops.cc:359).  For LORAX_A_RH the launch
+ * may write it (fp32 partial sums and arrival counters when K is split across workgroups: h_in not a multiple
+ * of 128 and a few hundred to a few thousand rows); nothing is expected in it on entry and nothing of value is
+ * left in it.  As in the reference, two shrinks that are in flight at the same time (different streams) must
+ * not share one tmp buffer.
  */
 int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
                       const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
@@ -255,15 +260,13 @@ int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t num_tokens,
                              int32_t group_capacity, int32_t* num_groups);
 
 /*
- * Allocates (once per device, idempotent) the library's workspace on `device`:
- * split-K partial sums and their arrival counters.  Call it outside graph capture
- * before the first SGMV shrink on a device; the reference has no counterpart because
- * its scratch arrives through `tmp` (punica.py:145-167).  Calls that use the
- * workspace concurrently on different streams of one device race.
+ * Per-device set-up.  Nothing is allocated: every entry point above takes its scratch from the caller, as the
+ * reference does (punica.py:145-167).  Kept so that a host can check a device index once at start-up; calling
+ * it is optional.
  */
 int lorax_init(int32_t device);
 
-/* Workspace bytes lorax_init reserves per device. */
+/* Device memory the library itself holds per GPU, in bytes. */
 size_t lorax_workspace_bytes(void);
 
 /* Message of the last error on this thread ("" if none).  Host pointer, valid until

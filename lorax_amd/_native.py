@@ -167,7 +167,7 @@ def _raise_last(rc: int):
 
 
 def init(device) -> None:
-    """Allocates the library's workspace on `device` (idempotent). Must not run under graph capture."""
+    """lorax_init: per-device set-up of the library (idempotent; call it outside graph capture)."""
     index = torch.device(device).index
     if index is None:
         index = torch.cuda.current_device()

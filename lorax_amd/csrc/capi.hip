@@ -1,11 +1,9 @@
-// C ABI of liblorax_hip.so: argument validation, error reporting, per-device
-// workspace and dispatch to the kernel launchers.  The checks mirror the TORCH_CHECKs
+// C ABI of liblorax_hip.so: argument validation, error reporting and dispatch to the kernel launchers.  The checks mirror the TORCH_CHECKs
 // of the reference's pybind layer (punica_kernels/punica_ops.cc:291-411); what that
 // layer reads from tensor metadata arrives here as plain integers.
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
-#include <mutex>
 
 #include "kernels.h"
 
@@ -14,13 +12,6 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 constexpr int kMaxRank = 128;  // BGMV_MAX_RANK / MAX_RANK_CUSTOM, punica.py:37-39
-
-struct Workspace {
-  float* partials = nullptr;
-  uint32_t* counters = nullptr;
-};
-Workspace g_ws[kMaxDevices];
-std::mutex g_ws_mutex;
 
 thread_local char g_error[512] = "";
 
@@ -34,51 +25,12 @@ int fail(int code, const char* fmt, ...) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+#ifdef LORAX_TUNING_ENV
 int env_int(const char* name) {
   const char* s = getenv(name);
   return s ? atoi(s) : 0;
 }
-
-int init_device(int device) {
-  if (device < 0 || device >= kMaxDevices) return fail(LORAX_EINVAL, "device %d out of range", device);
-  std::lock_guard<std::mutex> lock(g_ws_mutex);
-  if (g_ws[device].partials != nullptr) return LORAX_OK;
-  int prev = 0;
-  hipError_t e = hipGetDevice(&prev);
-  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
-  if (prev != device) {
-    e = hipSetDevice(device);
-    if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
-  }
-  float* partials = nullptr;
-  uint32_t* counters = nullptr;
-  e = hipMalloc(reinterpret_cast<void**>(&partials), kPartialBytes);
-  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&counters), kNumCounters * sizeof(uint32_t));
-  if (e == hipSuccess) e = hipMemset(counters, 0, kNumCounters * sizeof(uint32_t));
-  if (e == hipSuccess) e = hipDeviceSynchronize();
-  if (prev != device) (void)hipSetDevice(prev);
-  if (e != hipSuccess) {
-    if (partials) (void)hipFree(partials);
-    if (counters) (void)hipFree(counters);
-    return fail(LORAX_ELAUNCH, "workspace allocation on device %d: %s", device, hipGetErrorString(e));
-  }
-  g_ws[device].partials = partials;
-  g_ws[device].counters = counters;
-  return LORAX_OK;
-}
-
-// Workspace of the current device; allocates it on first use unless `stream` is
-// being captured (allocation is not a capturable operation).
-Workspace current_workspace(hipStream_t stream) {
-  int device = 0;
-  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return Workspace{};
-  if (g_ws[device].partials == nullptr) {
-    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &status) == hipSuccess && status == hipStreamCaptureStatusNone)
-      (void)init_device(device);
-  }
-  return g_ws[device];
-}
+#endif
 
 int check_common(const void* y, const void* x, const void* w_ptrs, int dtype) {
   if (y == nullptr || x == nullptr || w_ptrs == nullptr)
@@ -92,10 +44,16 @@ int check_common(const void* y, const void* x, const void* w_ptrs, int dtype) {
 
 }  // namespace
 
+// Launch parameters are the launchers' own heuristics in the product build; a tuning build
+// (-DLORAX_TUNING_ENV) lets LORAX_* environment variables override them, read once per process.
 const Tuning& tuning() {
+#ifndef LORAX_TUNING_ENV
+  static const Tuning t = {};
+#else
   static const Tuning t = {env_int("LORAX_BGMV_LORA_BLOCKS"), env_int("LORAX_BGMV_SHRINK_ROWS"), env_int("LORAX_SHRINK_KSPLIT"),
                            env_int("LORAX_SHRINK_MB"), env_int("LORAX_SHRINK_WAVES"), env_int("LORAX_EXPAND_ROWS"),
                            env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB"), env_int("LORAX_BGMV_EXPAND_COLS"), env_int("LORAX_EXPAND_PANELS"), env_int("LORAX_BGMV_NO_RUNS"), env_int("LORAX_BGMV_NO_BALANCE"), env_int("LORAX_SHRINK_ROWS_MAX")};
+#endif
   return t;
 }
 
@@ -220,14 +178,11 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
     return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p tmp=%p)", s_start, s_end, tmp);
   if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
   // [L, r, h_in]: multiples of 16 as in the reference (sgmv_config.h:10-15), and any multiple of 8 where the
-  // LDS-staged kernel (h_in a multiple of 128) or the streaming kernel (up to 512 rows) applies
-  const bool r_ok = r >= 8 && r <= kMaxRank && r % 8 == 0 &&
-                    (a_layout == LORAX_A_HR || r % 16 == 0 || h_in % 128 == 0 || num_tokens <= 512);
-  if (!r_ok || h_in <= 0 || h_in % 8 != 0 || num_tokens > INT32_MAX / 2)
+  // LDS-staged kernel or the streaming kernel applies (sgmv_shrink_route decides, below)
+  if (r < 8 || r > kMaxRank || r % 8 != 0 || h_in <= 0 || h_in % 8 != 0 || num_tokens > INT32_MAX / 2)
     return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in,
                 r, a_layout);
   const hipStream_t st = static_cast<hipStream_t>(stream);
-  const Workspace ws = current_workspace(st);
   SgmvArgs a{};
   a.y = v;
   a.x = x;
@@ -242,10 +197,16 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
   a.layer_idx = layer_idx;
   a.dtype = dtype;
   a.scale = scale;
-  a.partials = ws.partials;
-  a.partial_bytes = ws.partials ? kPartialBytes : 0;
-  a.counters = ws.counters;
-  a.num_counters = ws.counters ? kNumCounters : 0;
+  // Split-K scratch: the caller's 8 MiB buffer, as in the reference (sgmv_all.cu:10-65 takes its partial sums
+  // and its barrier words from tmp).  Its contents are never assumed: the counters are cleared by the launch.
+  if (a_layout == LORAX_A_RH && tmp != nullptr && aligned16(tmp)) {
+    a.partials = static_cast<float*>(tmp);
+    a.partial_bytes = kPartialBytes;
+    a.counters = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(tmp) + kPartialBytes);
+    a.num_counters = kNumCounters;
+  }
+  if (sgmv_shrink_route(a) == ShrinkRoute::kNone)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in, r, a_layout);
   const hipError_t e = launch_sgmv_shrink(a, st);
   if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_shrink launch failed: %s", hipGetErrorString(e));
   return LORAX_OK;
@@ -403,9 +364,12 @@ size_t lorax_sgmv_tmp_size(int32_t num_problems) {
   return num_problems > 0 ? static_cast<size_t>(num_problems) * (3 * 8 + 3 * 8 + 12) : 0;
 }
 
-int lorax_init(int32_t device) { return init_device(device); }
+int lorax_init(int32_t device) {
+  if (device < 0 || device >= kMaxDevices) return fail(LORAX_EINVAL, "device %d out of range", device);
+  return LORAX_OK;
+}
 
-size_t lorax_workspace_bytes(void) { return kPartialBytes + kNumCounters * sizeof(uint32_t); }
+size_t lorax_workspace_bytes(void) { return 0; }
 
 const char* lorax_last_error(void) { return g_error; }
 

@@ -89,7 +89,8 @@ struct SgmvArgs {
   ShrinkGroup group;  // shrink of several projections: count > 1, d_out = count * rank; else unused
   float scale;     // shrink: factor applied to the fp32 sums before rounding (1 in the reference's calls)
   int accumulate;  // expand: 1 = add to y (the reference's only mode), 0 = overwrite the rows of the segments
-  // library workspace of the current device (shrink split-K)
+  // scratch of the shrink's split-K (the caller's tmp, or the library's static array): fp32 partial tiles and one
+  // arrival counter per row tile; null = no scratch, the launch does not split K across workgroups
   float* partials;
   size_t partial_bytes;
   uint32_t* counters;
@@ -127,8 +128,25 @@ hipError_t launch_sgmv_shrink_lds(const SgmvArgs& a, hipStream_t stream);
 // Streaming shrink for a handful of rows (bgmv.hip): [L, r, h_in] layout, any h_in the BGMV kernels take.
 hipError_t launch_sgmv_shrink_rows(const SgmvArgs& a, hipStream_t stream);
 
-// Workspace layout constants shared by capi.hip and sgmv_shrink.hip.
-constexpr size_t kPartialBytes = 96u << 20;  // fp32 split-K partial sums
-constexpr size_t kNumCounters = 1u << 18;    // one arrival counter per row tile
+// Which kernel serves an SGMV shrink call (launch_sgmv_shrink dispatches on it; the C ABI derives from it
+// which shapes it accepts).
+enum class ShrinkRoute {
+  kNone,       // no kernel takes the shape
+  kRows,       // streaming kernel for a few hundred rows, [L, r, h_in]
+  kLds,        // LDS-staged MFMA kernel, [L, r, h_in], h_in a multiple of 128
+  kRegisters,  // register-operand MFMA kernel, [L, r, h_in], r a multiple of 16; the only one that may split K
+               // across workgroups and so the only one that touches the scratch
+  kNarrowRows  // [L, h_in, r] layout (rank 8 in the reference)
+};
+ShrinkRoute sgmv_shrink_route(const SgmvArgs& a);
+
+// Layout of the shrink scratch, the same inside the caller's 8 MiB tmp buffer and inside the library's static
+// array: fp32 partial tiles first, then the arrival counters.
+constexpr size_t kShrinkScratchBytes = 8u << 20;
+constexpr size_t kShrinkCounterBytes = 64u << 10;
+constexpr size_t kPartialBytes = kShrinkScratchBytes - kShrinkCounterBytes;
+constexpr size_t kNumCounters = kShrinkCounterBytes / sizeof(uint32_t);
+// K splits the register-operand shrink would use for this call given its scratch (1 = none).
+int sgmv_shrink_ksplit(const SgmvArgs& a);
 
 }  // namespace lorax

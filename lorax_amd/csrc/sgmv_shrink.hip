@@ -261,13 +261,64 @@ __global__ __launch_bounds__(256) void sgmv_shrink_hr_kernel(
   }
 }
 
+// Arrival counters must read zero when a split-K launch starts.  The last arrival of every tile resets its
+// counter, but the scratch may be a buffer nobody ever initialised (the caller's tmp) or may have been left
+// dirty by a launch that was torn down, so every split-K launch is preceded by this fill.  A kernel, not a
+// memset, so that the pair can be captured into a graph.
+__global__ void zero_counters_kernel(uint32_t* __restrict__ counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0u;
+}
+
 // ---------------------------------------------------------------------------------
 // Host-side launchers
 // ---------------------------------------------------------------------------------
+// Row-tile height (in 16-row blocks) of the register-operand kernel: 64 rows when there are many rows, 16 for
+// short batches so the few tiles there are do not carry padding; above rank 64 at most 32 rows (registers).
+static int rh_row_blocks(const SgmvArgs& a) {
+  const int nb = a.d_out / 16;
+  int mb = a.num_tokens >= 2048 ? 4 : (a.num_tokens >= 256 ? 2 : 1);
+  if (tuning().shrink_mb > 0) mb = tuning().shrink_mb;
+  if (mb != 1 && mb != 2 && mb != 4) mb = 1;
+  if (nb > 4 && mb > 2) mb = 2;
+  return mb;
+}
+
+// Splitting K across workgroups costs a device-scope fence per workgroup, which is only worth paying when the
+// row tiles alone cannot occupy the 256 CUs; the split is cut to what the scratch holds.
+int sgmv_shrink_ksplit(const SgmvArgs& a) {
+  const int mb = rh_row_blocks(a);
+  const int64_t tiles = (a.num_tokens + mb * 16 - 1) / (mb * 16) + a.num_segments;
+  const int ksteps = (a.d_in + 31) / 32;
+  int ksplit = 1;
+  if (tuning().shrink_ksplit > 0) {
+    ksplit = tuning().shrink_ksplit;
+  } else if (tiles < 192) {
+    const int64_t want = (384 + tiles - 1) / tiles;
+    const int kmax = ksteps / 16 > 0 ? ksteps / 16 : 1;
+    ksplit = static_cast<int>(want < kmax ? want : kmax);
+    if (ksplit > 8) ksplit = 8;
+  }
+  if (ksplit > ksteps) ksplit = ksteps;
+  if (ksplit < 1) ksplit = 1;
+  if (ksplit > 1) {
+    const size_t per_chunk = static_cast<size_t>(a.num_tokens) * a.d_out * sizeof(float);
+    const size_t fit = per_chunk ? a.partial_bytes / per_chunk : 1;
+    if (static_cast<size_t>(ksplit) > fit) ksplit = static_cast<int>(fit);
+    if (ksplit < 1) ksplit = 1;
+    if (static_cast<size_t>(tiles) > a.num_counters || a.partials == nullptr || a.counters == nullptr) ksplit = 1;
+  }
+  return ksplit;
+}
+
 template <typename D, int NB, int MB, int WAVES>
 static hipError_t launch_rh_w(const SgmvArgs& a, int ksplit, hipStream_t stream) {
   const int64_t tiles = (a.num_tokens + MB * 16 - 1) / (MB * 16) + a.num_segments;
   dim3 grid(ksplit, static_cast<unsigned>(tiles < 65535 ? tiles : 65535));
+  if (ksplit > 1) {
+    const int n = static_cast<int>(tiles);  // sgmv_shrink_ksplit: tiles <= num_counters whenever K is split
+    hipLaunchKernelGGL(zero_counters_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, a.counters, n);
+  }
   hipLaunchKernelGGL((sgmv_shrink_rh_kernel<D, NB, MB, WAVES>), grid, dim3(WAVES * kWave), 0,
                      stream, static_cast<typename D::E*>(a.y),
                      static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end,
@@ -288,36 +339,8 @@ static hipError_t launch_rh(const SgmvArgs& a, int ksplit, hipStream_t stream) {
 
 template <typename D, int NB>
 static hipError_t launch_rh_nb(const SgmvArgs& a, hipStream_t stream) {
-  // Row-tile height: 64 rows when there are many rows, 16 for short batches so the few
-  // tiles there are do not carry padding.
-  int mb = a.num_tokens >= 2048 ? 4 : (a.num_tokens >= 256 ? 2 : 1);
-  if (NB > 4 && mb > 2) mb = 2;  // keep the accumulators within the register budget
-  if (tuning().shrink_mb > 0) mb = tuning().shrink_mb;
-  if (mb != 1 && mb != 2 && mb != 4) mb = 1;
-  if (NB > 4 && mb > 2) mb = 2;
-
-  // Splitting K across workgroups costs a device-scope fence per workgroup, which is only worth
-  // paying when the row tiles alone cannot occupy the 256 CUs.
-  const int64_t tiles = (a.num_tokens + mb * 16 - 1) / (mb * 16) + a.num_segments;
-  const int ksteps = (a.d_in + 31) / 32;
-  int ksplit = 1;
-  if (tuning().shrink_ksplit > 0) {
-    ksplit = tuning().shrink_ksplit;
-  } else if (tiles < 192) {
-    const int64_t want = (384 + tiles - 1) / tiles;
-    const int kmax = ksteps / 16 > 0 ? ksteps / 16 : 1;
-    ksplit = static_cast<int>(want < kmax ? want : kmax);
-    if (ksplit > 8) ksplit = 8;
-  }
-  if (ksplit > ksteps) ksplit = ksteps;
-  if (ksplit < 1) ksplit = 1;
-  if (ksplit > 1) {
-    const size_t per_chunk = static_cast<size_t>(a.num_tokens) * NB * 16 * sizeof(float);
-    const size_t fit = per_chunk ? a.partial_bytes / per_chunk : 1;
-    if (static_cast<size_t>(ksplit) > fit) ksplit = static_cast<int>(fit);
-    if (ksplit < 1) ksplit = 1;
-    if (static_cast<size_t>(tiles) > a.num_counters || a.partials == nullptr) ksplit = 1;
-  }
+  const int mb = rh_row_blocks(a);
+  const int ksplit = sgmv_shrink_ksplit(a);
   if constexpr (NB <= 4) {
     if (mb == 4) return launch_rh<D, NB, 4>(a, ksplit, stream);
   }
@@ -337,6 +360,7 @@ static hipError_t launch_shrink_dtype(const SgmvArgs& a, hipStream_t stream) {
                        static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, a.scale);
     return hipGetLastError();
   }
+  if (a.d_out % 16 != 0) return hipErrorInvalidValue;  // the register-operand kernel works in 16-column blocks
   switch (a.d_out / 16) {
     case 1:
       return launch_rh_nb<D, 1>(a, stream);
@@ -359,17 +383,31 @@ static hipError_t launch_shrink_dtype(const SgmvArgs& a, hipStream_t stream) {
   }
 }
 
-hipError_t launch_sgmv_shrink(const SgmvArgs& a, hipStream_t stream) {
+ShrinkRoute sgmv_shrink_route(const SgmvArgs& a) {
+  if (a.d_out < 8 || a.d_out > 128 || a.d_out % 8 != 0 || a.d_in <= 0 || a.d_in % 8 != 0) return ShrinkRoute::kNone;
+  if (a.a_layout == LORAX_A_HR) return ShrinkRoute::kNarrowRows;
+  if (a.a_layout != LORAX_A_RH) return ShrinkRoute::kNone;
   // Up to a few hundred rows there are too few MFMA tiles to occupy the chip; the streaming kernel splits K
   // inside every workgroup instead of across workgroups (64 rows: 4.2 us against 10.4 us).
   const int rows_max = tuning().shrink_rows_max != 0 ? tuning().shrink_rows_max : 512;
-  if (a.a_layout == LORAX_A_RH && a.num_tokens <= rows_max && a.d_out % 8 == 0)
-    return launch_sgmv_shrink_rows(a, stream);
+  if (a.num_tokens <= rows_max) return ShrinkRoute::kRows;
   // The LDS-staged kernel is the faster one wherever it applies (h_in a multiple of 128).
-  if (tuning().shrink_lds >= 0 && sgmv_shrink_lds_applies(a))
-    return launch_sgmv_shrink_lds(a, stream);
-  return a.dtype == LORAX_F16 ? launch_shrink_dtype<F16>(a, stream)
-                              : launch_shrink_dtype<BF16>(a, stream);
+  if (tuning().shrink_lds >= 0 && sgmv_shrink_lds_applies(a)) return ShrinkRoute::kLds;
+  return a.d_out % 16 == 0 ? ShrinkRoute::kRegisters : ShrinkRoute::kNone;
+}
+
+hipError_t launch_sgmv_shrink(const SgmvArgs& a, hipStream_t stream) {
+  switch (sgmv_shrink_route(a)) {
+    case ShrinkRoute::kRows:
+      return launch_sgmv_shrink_rows(a, stream);
+    case ShrinkRoute::kLds:
+      return launch_sgmv_shrink_lds(a, stream);
+    case ShrinkRoute::kRegisters:
+    case ShrinkRoute::kNarrowRows:
+      return a.dtype == LORAX_F16 ? launch_shrink_dtype<F16>(a, stream) : launch_shrink_dtype<BF16>(a, stream);
+    default:
+      return hipErrorInvalidValue;
+  }
 }
 
 }  // namespace lorax

@@ -115,7 +115,7 @@ def test_sgmv_shrink_expand_vs_oracle(dtype, r, h_in, h_out, lens):
                        [torch.eye(r, dtype=dtype).expand(2, r, r) if w is not None else None for w in wb],
                        starts, ends, layer, r)
     y_ref = O.sgmv_ref(y0.cpu().clone(), x.cpu(), cpu(wa), cpu(wb), starts, ends, layer, r)
-    assert_close(v, v_ref, "shrink output v", max_abs=4e-2)  # |v| reaches 4..8 where one bf16 ulp is 0.031
+    assert_close(v, v_ref, "shrink output v")  # where |v| reaches 4..8 the limit is the spacing of the type there
     assert_close(y, y_ref, "expand output y")
     covered = torch.zeros(T, dtype=torch.bool)
     for s, e in zip(starts, ends):
@@ -340,22 +340,29 @@ def test_sgmv_expand_column_window():
     assert_close(y, y_ref, "fused gate/up output")
 
 
-def test_sgmv_split_k_is_deterministic_and_leaves_workspace_clean():
-    """Few row tiles and a long hidden dimension force the split-K path; repeated calls must give
-    bit-identical results (fixed summation order, counters reset by the last arrival)."""
-    dtype, r, h_in = torch.bfloat16, 64, 14336
-    gen = torch.Generator().manual_seed(9)
-    T, x, _, wa, _, starts, ends = _ragged_case(dtype, r, h_in, 8, [16, 5, 48], gen, gaps=True)
+@pytest.mark.parametrize("r,h_in,lens", [(16, 4160, [300, 7, 313]), (64, 2080, [520, 1, 40]), (128, 1056, [700])])
+def test_sgmv_split_k_is_deterministic_and_cleans_its_counters(r, h_in, lens):
+    """More than 512 rows, h_in not a multiple of 128 and few row tiles: the register-operand kernel with K split
+    across workgroups, partial sums and arrival counters in the caller's tmp.  The tmp buffer is filled with
+    garbage before every call (nothing may be expected in it), and repeated calls must give bit-identical results
+    (fixed summation order)."""
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(9 + r)
+    T, x, _, wa, _, starts, ends = _ragged_case(dtype, r, h_in, 8, lens, gen, gaps=True)
+    assert T > 512
     s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
     s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
     tmp = sgmv.get_tmp_tensor(x.device)
-    outs = [sgmv.lora_a_sgmv_cutlass(x, tmp, ptr_table(wa, DEV), s_start, s_end, 1, r) for _ in range(4)]
+    outs = []
+    for i in range(4):
+        tmp.fill_(0xA5 + i)
+        outs.append(sgmv.lora_a_sgmv_cutlass(x, tmp, ptr_table(wa, DEV), s_start, s_end, 1, r))
     torch.cuda.synchronize()
     for o in outs[1:]:
         assert torch.equal(o, outs[0])
     v_ref = O.sgmv_ref(torch.zeros((T, r), dtype=dtype), x.cpu(), [w.cpu() for w in wa],
-                       [torch.eye(r, dtype=dtype).expand(2, r, r)] * 3, starts, ends, 1, r)
-    assert_close(outs[0], v_ref, "v", max_abs=4e-2)
+                       [torch.eye(r, dtype=dtype).expand(2, r, r)] * len(lens), starts, ends, 1, r)
+    assert_close(outs[0], v_ref, "v")
 
 
 def test_sgmv_errors_raise_runtime_error():
