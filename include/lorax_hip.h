@@ -171,6 +171,26 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
                       void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
 
 /*
+ * lorax_sgmv_shrink without a tmp argument and without any allocation.  It has no counterpart in the reference;
+ * it is for callers that cannot allocate device memory or hand a scratch buffer over: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The result is bit-identical to
+ * lorax_sgmv_shrink's on the same arguments.  The split-K scratch is an array of LORAX_SHRINK_TMP_BYTES (8 MiB)
+ * inside the library's own device image, one copy per GPU, held until the process ends; its address on a
+ * device is looked up on the first call there (or by lorax_init).
+ *
+ * Limit: a call served by the split-K kernel (LORAX_A_RH, h_in not a multiple of 128, more than 512 rows) needs
+ * 2 * num_tokens * r * 4 bytes <= LORAX_SHRINK_TMP_BYTES - 65536, i.e. room for two fp32 partial tiles of the
+ * batch; beyond that the call fails with LORAX_ESPACE and launches nothing.  Other shapes use no scratch and
+ * have no limit.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * streams or threads) race; calls on one stream, or ordered by events, do not.  Nothing needs to be cleared
+ * between calls (the arrival counters are cleared by every launch that uses them).
+ */
+int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
+                             const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t h_in,
+                             int32_t r, int32_t a_layout, int64_t layer_idx, float scale, int32_t dtype,
+                             void* stream);
+
+/*
  * SGMV shrink of up to 4 projections that share x, the segments and the rank (q/k/v, gate/up), LORAX_A_RH
  * stacks: problem p gets v_p[s:e, :] += dtype(scale * x[s:e, :] @ A_p^T) exactly as from lorax_sgmv_shrink
  * with (v_p, w_ptrs_p).  The reference launches one shrink per projection (lorax_server/utils/layers.py:
@@ -260,13 +280,13 @@ int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t num_tokens,
                              int32_t group_capacity, int32_t* num_groups);
 
 /*
- * Per-device set-up.  Nothing is allocated: every entry point above takes its scratch from the caller, as the
- * reference does (punica.py:145-167).  Kept so that a host can check a device index once at start-up; calling
- * it is optional.
+ * Per-device set-up: looks up the address of the static scratch of lorax_sgmv_shrink_static on `device`.
+ * Nothing is allocated (every other entry point takes its scratch from the caller, as the reference does,
+ * punica.py:145-167).  Optional: lorax_sgmv_shrink_static does the same on its first call on a device.
  */
 int lorax_init(int32_t device);
 
-/* Device memory the library itself holds per GPU, in bytes. */
+/* Device memory the library itself holds per GPU, in bytes (the static scratch). */
 size_t lorax_workspace_bytes(void);
 
 /* Message of the last error on this thread ("" if none).  Host pointer, valid until

@@ -89,6 +89,11 @@ _SIGNATURES = {
          _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_void_p, _c.c_int64, _c.c_int32,
          _c.c_void_p],
     ),
+    "lorax_sgmv_shrink_static": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
+         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_int32, _c.c_void_p],
+    ),
     "lorax_sgmv_shrink_multi": (
         _c.c_int,
         [_c.POINTER(SgmvShrinkProblem), _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
@@ -401,6 +406,19 @@ def sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, scale: float = 1.0)
     if isinstance(tmp, torch.Tensor) and tmp.dtype != torch.uint8:
         raise RuntimeError(f"CHECK_EQ(tmp.scalar_type(), at::ScalarType::Byte) failed. {tmp.dtype}")
     return _sgmv_shrink(y, x, w_ptr, s_start, s_end, tmp, layer_idx, A_RH, scale)
+
+
+def sgmv_shrink_static(y, x, w_ptr, s_start, s_end, layer_idx, a_layout=A_RH, scale: float = 1.0) -> None:
+    """lorax_sgmv_shrink_static: sgmv_shrink / the shrink direction of sgmv_cutlass without a tmp tensor; the
+    library's own static device array serves as split-K scratch, so the call allocates nothing."""
+    _check_sgmv(y, x, w_ptr, s_start, s_end, s_start)
+    with torch.cuda.device(x.device):
+        rc = lib().lorax_sgmv_shrink_static(
+            y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0),
+            x.size(0), x.size(1), y.size(1), a_layout, int(layer_idx), float(scale), _dtype_code(x), _stream(x),
+        )
+    if rc != 0:
+        _raise_last(rc)
 
 
 MAX_SGMV_SHRINK_PROBLEMS = 4

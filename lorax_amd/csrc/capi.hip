@@ -1,6 +1,7 @@
 // C ABI of liblorax_hip.so: argument validation, error reporting and dispatch to the kernel launchers.  The checks mirror the TORCH_CHECKs
 // of the reference's pybind layer (punica_kernels/punica_ops.cc:291-411); what that
 // layer reads from tensor metadata arrives here as plain integers.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -12,6 +13,14 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 constexpr int kMaxRank = 128;  // BGMV_MAX_RANK / MAX_RANK_CUSTOM, punica.py:37-39
+
+// Scratch of lorax_sgmv_shrink_static: device memory that exists from the moment the library is loaded, so that
+// entry point never allocates.  Same layout as the caller's tmp of lorax_sgmv_shrink (kernels.h).  Every GPU
+// holds its own copy at its own address; in host code the array's name is only a handle for the runtime (passed
+// to a kernel it would be a host address and the kernel would fault), so the device address is asked for once
+// per device and kept.
+static __device__ __align__(256) unsigned char scratch[kShrinkScratchBytes];
+std::atomic<unsigned char*> g_scratch_ptr[kMaxDevices];
 
 thread_local char g_error[512] = "";
 
@@ -31,6 +40,31 @@ int env_int(const char* name) {
   return s ? atoi(s) : 0;
 }
 #endif
+
+// Address of `scratch` on `device`, asked for on first use with that device current.  Two threads that race here
+// ask twice and store the same address, which is harmless.
+int resolve_scratch(int device, unsigned char** out) {
+  if (device < 0 || device >= kMaxDevices) return fail(LORAX_EINVAL, "device %d out of range", device);
+  unsigned char* p = g_scratch_ptr[device].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    int prev = 0;
+    hipError_t e = hipGetDevice(&prev);
+    if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (prev != device) {
+      e = hipSetDevice(device);
+      if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
+    }
+    void* addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (prev != device) (void)hipSetDevice(prev);
+    if (e != hipSuccess || addr == nullptr)
+      return fail(LORAX_ELAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", device, hipGetErrorString(e));
+    p = static_cast<unsigned char*>(addr);
+    g_scratch_ptr[device].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return LORAX_OK;
+}
 
 int check_common(const void* y, const void* x, const void* w_ptrs, int dtype) {
   if (y == nullptr || x == nullptr || w_ptrs == nullptr)
@@ -134,6 +168,57 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
   return LORAX_OK;
 }
 
+// Shape checks and launch shared by lorax_sgmv_shrink and lorax_sgmv_shrink_static.  `scratch_buf` is
+// kShrinkScratchBytes of device memory (partial tiles, then arrival counters) or null.  With `must_fit`, a call
+// that is served by the split-K kernel is refused unless the scratch holds two fp32 partial tiles of the batch.
+int sgmv_shrink_checked(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start, const int32_t* s_end,
+                        int32_t num_segments, int64_t num_tokens, int32_t h_in, int32_t r, int32_t a_layout,
+                        int64_t layer_idx, float scale, void* scratch_buf, bool must_fit, int32_t dtype, void* stream) {
+  if (int rc = check_common(v, x, w_ptrs, dtype)) return rc;
+  if (s_start == nullptr || s_end == nullptr)
+    return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p)", s_start, s_end);
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  // [L, r, h_in]: multiples of 16 as in the reference (sgmv_config.h:10-15), and any multiple of 8 where the
+  // LDS-staged kernel or the streaming kernel applies (sgmv_shrink_route decides, below)
+  if (r < 8 || r > kMaxRank || r % 8 != 0 || h_in <= 0 || h_in % 8 != 0 || num_tokens > INT32_MAX / 2)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in,
+                r, a_layout);
+  SgmvArgs a{};
+  a.y = v;
+  a.x = x;
+  a.w_ptrs = w_ptrs;
+  a.s_start = s_start;
+  a.s_end = s_end;
+  a.num_segments = num_segments;
+  a.num_tokens = num_tokens;
+  a.d_in = h_in;
+  a.d_out = r;
+  a.a_layout = a_layout;
+  a.layer_idx = layer_idx;
+  a.dtype = dtype;
+  a.scale = scale;
+  if (scratch_buf != nullptr) {
+    a.partials = static_cast<float*>(scratch_buf);
+    a.partial_bytes = kPartialBytes;
+    a.counters = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(scratch_buf) + kPartialBytes);
+    a.num_counters = kNumCounters;
+  }
+  const ShrinkRoute route = sgmv_shrink_route(a);
+  if (route == ShrinkRoute::kNone)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in, r, a_layout);
+  if (must_fit && route == ShrinkRoute::kRegisters) {
+    const int64_t need = 2 * num_tokens * r * static_cast<int64_t>(sizeof(float));
+    if (need > static_cast<int64_t>(kPartialBytes))
+      return fail(LORAX_ESPACE,
+                  "batch too large for the static scratch: 2 * num_tokens * r * 4 = %lld bytes, limit %zu "
+                  "(num_tokens=%lld r=%d); call lorax_sgmv_shrink with a tmp buffer instead",
+                  (long long)need, kPartialBytes, (long long)num_tokens, r);
+  }
+  const hipError_t e = launch_sgmv_shrink(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_shrink launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -173,43 +258,31 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
     return fail(LORAX_EINVAL, "a_layout=%d (0 = [L,r,h_in], 1 = [L,h_in,r])", a_layout);
   }
   if (num_segments == 0 || num_tokens == 0) return LORAX_OK;
-  if (int rc = check_common(v, x, w_ptrs, dtype)) return rc;
-  if (s_start == nullptr || s_end == nullptr || (tmp == nullptr && tmp_bytes > 0))
-    return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p tmp=%p)", s_start, s_end, tmp);
-  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
-  // [L, r, h_in]: multiples of 16 as in the reference (sgmv_config.h:10-15), and any multiple of 8 where the
-  // LDS-staged kernel or the streaming kernel applies (sgmv_shrink_route decides, below)
-  if (r < 8 || r > kMaxRank || r % 8 != 0 || h_in <= 0 || h_in % 8 != 0 || num_tokens > INT32_MAX / 2)
-    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in,
-                r, a_layout);
-  const hipStream_t st = static_cast<hipStream_t>(stream);
-  SgmvArgs a{};
-  a.y = v;
-  a.x = x;
-  a.w_ptrs = w_ptrs;
-  a.s_start = s_start;
-  a.s_end = s_end;
-  a.num_segments = num_segments;
-  a.num_tokens = num_tokens;
-  a.d_in = h_in;
-  a.d_out = r;
-  a.a_layout = a_layout;
-  a.layer_idx = layer_idx;
-  a.dtype = dtype;
-  a.scale = scale;
+  if (tmp == nullptr && tmp_bytes > 0) return fail(LORAX_EINVAL, "null pointer argument (tmp)");
   // Split-K scratch: the caller's 8 MiB buffer, as in the reference (sgmv_all.cu:10-65 takes its partial sums
   // and its barrier words from tmp).  Its contents are never assumed: the counters are cleared by the launch.
-  if (a_layout == LORAX_A_RH && tmp != nullptr && aligned16(tmp)) {
-    a.partials = static_cast<float*>(tmp);
-    a.partial_bytes = kPartialBytes;
-    a.counters = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(tmp) + kPartialBytes);
-    a.num_counters = kNumCounters;
-  }
-  if (sgmv_shrink_route(a) == ShrinkRoute::kNone)
-    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in, r, a_layout);
-  const hipError_t e = launch_sgmv_shrink(a, st);
-  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_shrink launch failed: %s", hipGetErrorString(e));
-  return LORAX_OK;
+  void* scratch_buf = (a_layout == LORAX_A_RH && aligned16(tmp)) ? tmp : nullptr;
+  return sgmv_shrink_checked(v, x, w_ptrs, s_start, s_end, num_segments, num_tokens, h_in, r, a_layout, layer_idx,
+                             scale, scratch_buf, false, dtype, stream);
+}
+
+int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
+                             const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t h_in,
+                             int32_t r, int32_t a_layout, int64_t layer_idx, float scale, int32_t dtype,
+                             void* stream) {
+  if (num_segments < 0 || num_tokens < 0)
+    return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments,
+                (long long)num_tokens);
+  if (a_layout != LORAX_A_RH && a_layout != LORAX_A_HR)
+    return fail(LORAX_EINVAL, "a_layout=%d (0 = [L,r,h_in], 1 = [L,h_in,r])", a_layout);
+  if (num_segments == 0 || num_tokens == 0) return LORAX_OK;
+  int device = 0;
+  const hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  unsigned char* buf = nullptr;
+  if (int rc = resolve_scratch(device, &buf)) return rc;
+  return sgmv_shrink_checked(v, x, w_ptrs, s_start, s_end, num_segments, num_tokens, h_in, r, a_layout, layer_idx,
+                             scale, buf, true, dtype, stream);
 }
 
 int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t num_problems, const void* x,
@@ -365,11 +438,11 @@ size_t lorax_sgmv_tmp_size(int32_t num_problems) {
 }
 
 int lorax_init(int32_t device) {
-  if (device < 0 || device >= kMaxDevices) return fail(LORAX_EINVAL, "device %d out of range", device);
-  return LORAX_OK;
+  unsigned char* p = nullptr;
+  return resolve_scratch(device, &p);
 }
 
-size_t lorax_workspace_bytes(void) { return 0; }
+size_t lorax_workspace_bytes(void) { return kShrinkScratchBytes; }
 
 const char* lorax_last_error(void) { return g_error; }
 
