@@ -168,10 +168,12 @@ class Plan:
         bt_ptr = rd.lora_b_t_ptr if fused else None
         a_is_rh = resident_a or not sgmv.use_cutlass_shrink(r)
         if a_is_rh:
-            tmp_s = sgmv.get_tmp_tensor(x.device)
+            tmp_s = sgmv.get_shrink_scratch(x.device) if resident_a else sgmv.get_tmp_tensor(x.device)
 
         def shrink(layer):
-            if a_is_rh:
+            if resident_a:
+                sgmv._kernels.sgmv_shrink_multi([v], x, [a_ptr], starts, ends, tmp_s, layer)
+            elif a_is_rh:
                 sgmv._kernels.sgmv_shrink(v, x, a_ptr, starts, ends, tmp_s, layer)
             else:
                 sgmv._kernels.sgmv_cutlass(v, x, a_ptr, starts, ends, tmp_s, layer)
@@ -203,7 +205,7 @@ class Plan:
         flat = torch.zeros((len(jobs), x.size(0), r), dtype=x.dtype, device=x.device)
         vs = list(flat.unbind(0))
         tables = [rd.lora_a_t_ptr for rd, _, _ in jobs]
-        tmp_s = sgmv.get_tmp_tensor(x.device)
+        tmp_s = sgmv.get_shrink_scratch(x.device)
         shrink_bytes = shrink_gather = rows * h_in * e
         for rd, _, _ in jobs:
             uniq = len(set(rd.lora_a_t_ptr[lens > 0].tolist()))

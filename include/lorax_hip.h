@@ -197,7 +197,9 @@ int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, cons
  * 121-133, punica_ops.cc:369-411) and reads x once per launch; here, when num_problems * r <= 128, h_in is a
  * multiple of 128 and the batch has more than 512 rows, the projections run as ONE launch that reads x once
  * (their A matrices are stacked into one rank-(num_problems * r) tile).  Otherwise the call issues one
- * launch per projection.  `tmp`/`tmp_bytes` as for lorax_sgmv_shrink with LORAX_A_RH.
+ * launch per projection.  `tmp`/`tmp_bytes`: at least LORAX_SHRINK_TMP_BYTES of scratch, as for lorax_sgmv_shrink
+ * with LORAX_A_RH; a larger buffer is accepted (a launch that splits K across workgroups keeps its fp32 partial
+ * sums there and can split further the more room it has).  num_problems = 1 is allowed.
  */
 typedef struct {
   void* v;               /* [num_tokens, r] */

@@ -295,20 +295,23 @@ int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t
   // One launch where the LDS-staged kernel takes the stacked rank and the batch is past the streaming
   // kernel's range; otherwise one launch per projection, with the same result.
   const int rows_max = tuning().shrink_rows_max != 0 ? tuning().shrink_rows_max : 512;
-  const bool stacked = num_problems > 1 && r >= 8 && r % 8 == 0 && num_problems * r <= kMaxRank && h_in > 0 &&
+  const bool stacked = r >= 8 && r % 8 == 0 && num_problems * r <= kMaxRank && h_in > 0 &&
                        h_in % 128 == 0 && num_tokens > rows_max && tuning().shrink_lds >= 0;
   if (!stacked) {
     for (int i = 0; i < num_problems; ++i) {
+      if (tmp_bytes < LORAX_SHRINK_TMP_BYTES)
+        return fail(LORAX_ETMPSIZE, "CHECK_GE(tmp.size(0), 8 * 1024 * 1024) failed. %lld vs %d", (long long)tmp_bytes,
+                    LORAX_SHRINK_TMP_BYTES);
       const int rc = lorax_sgmv_shrink(problems[i].v, x, problems[i].w_ptrs, s_start, s_end, num_segments, num_tokens,
-                                       h_in, r, LORAX_A_RH, layer_idx, scale, tmp, tmp_bytes, dtype, stream);
+                                       h_in, r, LORAX_A_RH, layer_idx, scale, tmp, LORAX_SHRINK_TMP_BYTES, dtype, stream);
       if (rc != LORAX_OK) return rc;
     }
     return LORAX_OK;
   }
   if (num_segments < 0 || num_tokens < 0)
     return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments, (long long)num_tokens);
-  if (tmp_bytes != LORAX_SHRINK_TMP_BYTES)
-    return fail(LORAX_ETMPSIZE, "CHECK_EQ(tmp.size(0), 8 * 1024 * 1024) failed. %lld vs %d", (long long)tmp_bytes,
+  if (tmp_bytes < LORAX_SHRINK_TMP_BYTES)
+    return fail(LORAX_ETMPSIZE, "CHECK_GE(tmp.size(0), 8 * 1024 * 1024) failed. %lld vs %d", (long long)tmp_bytes,
                 LORAX_SHRINK_TMP_BYTES);
   if (num_segments == 0) return LORAX_OK;
   for (int i = 0; i < num_problems; ++i)
@@ -332,6 +335,10 @@ int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t
   a.layer_idx = layer_idx;
   a.dtype = dtype;
   a.scale = scale;
+  if (aligned16(tmp)) {  // fp32 partial tiles of a launch that splits K
+    a.partials = static_cast<float*>(tmp);
+    a.partial_bytes = static_cast<size_t>(tmp_bytes);
+  }
   a.group.count = num_problems;
   a.group.rank = r;
   for (int i = 0; i < num_problems; ++i) {

@@ -30,7 +30,7 @@ from lorax_amd.adapters import LORA, AdapterBatchData, BatchLoraWeights
 from lorax_amd._native import MAX_SGMV_SHRINK_PROBLEMS
 from lorax_amd.sgmv import (
     MAX_RANK_CUSTOM,
-    get_tmp_tensor,
+    get_shrink_scratch,
     has_sgmv,
     lora_a_sgmv_cutlass,
     lora_a_sgmv_resident,
@@ -117,7 +117,7 @@ class LoraLinear(nn.Module):
                         prefill_jobs[(r, rs.segments_key)].append((rs, start, end - start))
                         continue
                     v = lora_a_sgmv_resident(
-                        input, get_tmp_tensor(input.device), rs.lora_a_t_ptr, rs.segment_starts, rs.segment_ends,
+                        input, get_shrink_scratch(input.device), rs.lora_a_t_ptr, rs.segment_starts, rs.segment_ends,
                         self.layer_id, r,
                     )
                 else:
@@ -150,7 +150,7 @@ class LoraLinear(nn.Module):
                 chunk = group[i : i + step]
                 first = chunk[0][0]
                 vs = lora_a_sgmv_resident_multi(
-                    input, get_tmp_tensor(input.device), [rs.lora_a_t_ptr for rs, _, _ in chunk],
+                    input, get_shrink_scratch(input.device), [rs.lora_a_t_ptr for rs, _, _ in chunk],
                     first.segment_starts, first.segment_ends, self.layer_id, r,
                 )
                 for v, (rs, start, width) in zip(vs, chunk):

@@ -95,6 +95,18 @@ def get_tmp_tensor(device: torch.device) -> torch.Tensor:
     return torch.empty((_SHRINK_TMP_BYTES,), dtype=torch.uint8, device=device)
 
 
+_RESIDENT_SCRATCH_BYTES = 32 * 1024 * 1024
+
+
+@lru_cache(maxsize=1)
+def get_shrink_scratch(device: torch.device) -> torch.Tensor:
+    """Scratch of the resident-layout shrink entries (lora_a_sgmv_resident, lora_a_sgmv_resident_multi): where a
+    batch has fewer row tiles than the GPU has CUs, K is split across workgroups and the fp32 partial sums
+    (splits x rows x summed rank) go here.  The reference's 8 MiB buffer (get_tmp_tensor) is accepted too and
+    only limits how far such a launch can split."""
+    return torch.empty((_RESIDENT_SCRATCH_BYTES,), dtype=torch.uint8, device=device)
+
+
 def get_tmp_expand_size(size: int) -> int:
     """punica.py:156-157."""
     return _native_module().sgmv_cutlass_tmp_size(size)
@@ -143,9 +155,9 @@ def lora_a_sgmv_resident(
     lora_rank: int,
 ) -> torch.Tensor:
     """As lora_a_sgmv_cutlass, reading the [L, r, h_in] stacks of the decode path (weights_a_t) whatever
-    the rank.  `tmp` is the 8 MiB buffer of get_tmp_tensor."""
+    the rank.  `tmp` is get_shrink_scratch(device) or the 8 MiB buffer of get_tmp_tensor."""
     v = torch.zeros((x.size(0), lora_rank), dtype=x.dtype, device=x.device)
-    _native_module().sgmv_shrink(v, x, wa_t_ptr, s_start, s_end, tmp, layer_idx)
+    _native_module().sgmv_shrink_multi([v], x, [wa_t_ptr], s_start, s_end, tmp, layer_idx)
     return v
 
 
