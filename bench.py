@@ -80,9 +80,9 @@ class Plan:
     static v and y buffers, and closures that issue the launches of ONE layer in order.
 
     pattern "fused" is what lorax_amd.layers issues: in decode one batched shrink launch and one batched
-    expand launch per projection group and rank (the shrink overwrites v, no zero-fill); in prefill a
-    zero-fill and a shrink per projection group and rank (up to a summed rank of 128 per launch) and an
-    expand per projection and rank.  pattern "reference" is the reference
+    expand launch per projection group and rank; in prefill a shrink per projection group and rank (up to a
+    summed rank of 128 per launch) and an expand per projection and rank.  The shrinks overwrite v, so there
+    is no zero-fill in either.  pattern "reference" is the reference
     caller's sequence (utils/layers.py:114-164): zero-fill, shrink, expand for every projection and rank.
     """
 
@@ -171,8 +171,8 @@ class Plan:
             tmp_s = sgmv.get_shrink_scratch(x.device) if resident_a else sgmv.get_tmp_tensor(x.device)
 
         def shrink(layer):
-            if resident_a:
-                sgmv._kernels.sgmv_shrink_multi([v], x, [a_ptr], starts, ends, tmp_s, layer)
+            if resident_a:  # overwrites the segments' rows of v: no zero-fill in this pattern
+                sgmv._kernels.sgmv_shrink_multi([v], x, [a_ptr], starts, ends, tmp_s, layer, 1.0, False)
             elif a_is_rh:
                 sgmv._kernels.sgmv_shrink(v, x, a_ptr, starts, ends, tmp_s, layer)
             else:
@@ -184,15 +184,16 @@ class Plan:
             else:
                 sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_ptr, starts, ends, layer, off, size)
 
-        self.calls.append(("zero", lambda layer: v.zero_(), 0, 0, 0))
+        if not resident_a:
+            self.calls.append(("zero", lambda layer: v.zero_(), 0, 0, 0))
         self.calls.append(("sgmv_shrink", shrink, rows * h_in * e + uniq * r * h_in * e + rows * r * e,
                            2 * rows * r * h_in, rows * h_in * e + rows * r * h_in * e + rows * r * e))
         self.calls.append(("sgmv_expand", expand, rows * r * e + uniq * r * size * e + 2 * rows * size * e,
                            2 * rows * r * size, rows * r * e + rows * r * size * e + 2 * rows * size * e))
 
     def _add_sgmv_group(self, x, y, h_in, r, jobs):
-        """Zero-fill and shrink of up to four projections in one launch each (x counted once), then one
-        expand per projection from the resident B^T stacks."""
+        """Shrink of up to four projections in one launch (x counted once; it overwrites v, no zero-fill), then
+        one expand per projection from the resident B^T stacks."""
         import torch
 
         from lorax_amd import _native, sgmv
@@ -211,9 +212,8 @@ class Plan:
             uniq = len(set(rd.lora_a_t_ptr[lens > 0].tolist()))
             shrink_bytes += uniq * r * h_in * e + rows * r * e
             shrink_gather += rows * r * h_in * e + rows * r * e
-        self.calls.append(("zero", lambda layer: flat.zero_(), 0, 0, 0))
         self.calls.append(("sgmv_shrink",
-                           lambda layer: _native.sgmv_shrink_multi(vs, x, tables, starts, ends, tmp_s, layer),
+                           lambda layer: _native.sgmv_shrink_multi(vs, x, tables, starts, ends, tmp_s, layer, 1.0, False),
                            shrink_bytes, 2 * rows * r * h_in * len(jobs), shrink_gather))
         for v, (rd, off, size) in zip(vs, jobs):
             uniq = len(set(rd.lora_b_t_ptr[lens > 0].tolist()))

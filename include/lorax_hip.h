@@ -200,6 +200,9 @@ int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, cons
  * launch per projection.  `tmp`/`tmp_bytes`: at least LORAX_SHRINK_TMP_BYTES of scratch, as for lorax_sgmv_shrink
  * with LORAX_A_RH; a larger buffer is accepted (a launch that splits K across workgroups keeps its fp32 partial
  * sums there and can split further the more room it has).  num_problems = 1 is allowed.
+ * accumulate = 1 adds to v as lorax_sgmv_shrink does; accumulate = 0 stores dtype(scale * x @ A^T) into the rows
+ * of the segments instead, so the caller need not zero v first (rows outside every segment keep their contents;
+ * lorax_sgmv_expand reads no others).  The reference zero-fills v before every shrink (punica.py:176-178).
  */
 typedef struct {
   void* v;               /* [num_tokens, r] */
@@ -209,7 +212,7 @@ typedef struct {
 int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t num_problems, const void* x,
                             const int32_t* s_start, const int32_t* s_end, int32_t num_segments,
                             int64_t num_tokens, int32_t h_in, int32_t r, int64_t layer_idx, float scale,
-                            void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
+                            int32_t accumulate, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
 
 /*
  * SGMV expand.  Replaces the expand direction of sgmv_cutlass (punica_ops.cc:338-367,

@@ -97,7 +97,8 @@ _SIGNATURES = {
     "lorax_sgmv_shrink_multi": (
         _c.c_int,
         [_c.POINTER(SgmvShrinkProblem), _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
-         _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_void_p, _c.c_int64, _c.c_int32, _c.c_void_p],
+         _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_int32, _c.c_void_p, _c.c_int64, _c.c_int32,
+         _c.c_void_p],
     ),
     "lorax_sgmv_expand": (
         _c.c_int,
@@ -424,9 +425,11 @@ def sgmv_shrink_static(y, x, w_ptr, s_start, s_end, layer_idx, a_layout=A_RH, sc
 MAX_SGMV_SHRINK_PROBLEMS = 4
 
 
-def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: float = 1.0) -> None:
+def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: float = 1.0,
+                      accumulate: bool = True) -> None:
     """lorax_sgmv_shrink_multi: sgmv_shrink for up to 4 projections (outputs `ys`, pointer tables `w_ptrs`) that
-    share x, the segment tables and the rank; one launch that reads x once where the kernels allow it."""
+    share x, the segment tables and the rank; one launch that reads x once where the kernels allow it.
+    accumulate=False overwrites the rows of the segments (no zero-fill of the outputs needed)."""
     if not 1 <= len(ys) <= MAX_SGMV_SHRINK_PROBLEMS or len(ys) != len(w_ptrs):
         raise RuntimeError(f"between 1 and {MAX_SGMV_SHRINK_PROBLEMS} outputs with one pointer table each")
     if isinstance(tmp, torch.Tensor) and tmp.dtype != torch.uint8:
@@ -442,8 +445,8 @@ def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: floa
     with torch.cuda.device(x.device):
         rc = lib().lorax_sgmv_shrink_multi(
             arr, len(ys), x.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0), x.size(0), x.size(1),
-            ys[0].size(1), int(layer_idx), float(scale), tmp.data_ptr(), tmp.numel() * tmp.element_size(),
-            _dtype_code(x), _stream(x),
+            ys[0].size(1), int(layer_idx), float(scale), 1 if accumulate else 0, tmp.data_ptr(),
+            tmp.numel() * tmp.element_size(), _dtype_code(x), _stream(x),
         )
     if rc != 0:
         _raise_last(rc)

@@ -200,9 +200,10 @@ template <typename D, int RS>
 __global__ __launch_bounds__(kBgmvThreads) void sgmv_shrink_rows_kernel(
     typename D::E* __restrict__ V, const typename D::E* __restrict__ X, const int64_t* __restrict__ W,
     const int32_t* __restrict__ s_start, const int32_t* __restrict__ s_end, int num_segments, int num_tokens,
-    int h_in, int r, int64_t layer_idx, float scale) {
+    int h_in, int r, int64_t layer_idx, float scale, int accumulate_into_v) {
   __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<RS * kGroup>::value];
   using E = typename D::E;
+  const bool acc_v = accumulate_into_v != 0;
   const int subs = r / RS;
   const int v = static_cast<int>(xcd_virtual_id());
   const int chunk = v / subs;
@@ -216,16 +217,16 @@ __global__ __launch_bounds__(kBgmvThreads) void sgmv_shrink_rows_kernel(
   const E* A = reinterpret_cast<const E*>(W[rt.seg]) + (layer_idx * r + row0) * static_cast<int64_t>(h_in);
   switch (n) {
     case 1:
-      bgmv_shrink_body<D, RS, 1>(V, X, A, toks, h_in, row0, 0, r, scale, true, red);
+      bgmv_shrink_body<D, RS, 1>(V, X, A, toks, h_in, row0, 0, r, scale, acc_v, red);
       break;
     case 2:
-      bgmv_shrink_body<D, RS, 2>(V, X, A, toks, h_in, row0, 0, r, scale, true, red);
+      bgmv_shrink_body<D, RS, 2>(V, X, A, toks, h_in, row0, 0, r, scale, acc_v, red);
       break;
     case 3:
-      bgmv_shrink_body<D, RS, 3>(V, X, A, toks, h_in, row0, 0, r, scale, true, red);
+      bgmv_shrink_body<D, RS, 3>(V, X, A, toks, h_in, row0, 0, r, scale, acc_v, red);
       break;
     default:
-      bgmv_shrink_body<D, RS, 4>(V, X, A, toks, h_in, row0, 0, r, scale, true, red);
+      bgmv_shrink_body<D, RS, 4>(V, X, A, toks, h_in, row0, 0, r, scale, acc_v, red);
       break;
   }
 }
@@ -238,7 +239,7 @@ static hipError_t launch_shrink_rows_dtype(const SgmvArgs& a, hipStream_t stream
   auto args = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(kBgmvThreads), 0, stream, static_cast<typename D::E*>(a.y),
                        static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end, a.num_segments,
-                       static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, a.scale);
+                       static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, a.scale, a.accumulate);
   };
   if (rs == 8) args(sgmv_shrink_rows_kernel<D, 8>);
   else if (rs == 4) args(sgmv_shrink_rows_kernel<D, 4>);

@@ -173,7 +173,10 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
 // that is served by the split-K kernel is refused unless the scratch holds two fp32 partial tiles of the batch.
 int sgmv_shrink_checked(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start, const int32_t* s_end,
                         int32_t num_segments, int64_t num_tokens, int32_t h_in, int32_t r, int32_t a_layout,
-                        int64_t layer_idx, float scale, void* scratch_buf, bool must_fit, int32_t dtype, void* stream) {
+                        int64_t layer_idx, float scale, int32_t accumulate, void* scratch_buf, bool must_fit,
+                        int32_t dtype, void* stream) {
+  if (accumulate != 0 && accumulate != 1)
+    return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (int rc = check_common(v, x, w_ptrs, dtype)) return rc;
   if (s_start == nullptr || s_end == nullptr)
     return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p)", s_start, s_end);
@@ -197,6 +200,7 @@ int sgmv_shrink_checked(void* v, const void* x, const int64_t* w_ptrs, const int
   a.layer_idx = layer_idx;
   a.dtype = dtype;
   a.scale = scale;
+  a.accumulate = accumulate;
   if (scratch_buf != nullptr) {
     a.partials = static_cast<float*>(scratch_buf);
     a.partial_bytes = kPartialBytes;
@@ -263,7 +267,7 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
   // and its barrier words from tmp).  Its contents are never assumed: the counters are cleared by the launch.
   void* scratch_buf = (a_layout == LORAX_A_RH && aligned16(tmp)) ? tmp : nullptr;
   return sgmv_shrink_checked(v, x, w_ptrs, s_start, s_end, num_segments, num_tokens, h_in, r, a_layout, layer_idx,
-                             scale, scratch_buf, false, dtype, stream);
+                             scale, 1, scratch_buf, false, dtype, stream);
 }
 
 int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
@@ -282,13 +286,15 @@ int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, cons
   unsigned char* buf = nullptr;
   if (int rc = resolve_scratch(device, &buf)) return rc;
   return sgmv_shrink_checked(v, x, w_ptrs, s_start, s_end, num_segments, num_tokens, h_in, r, a_layout, layer_idx,
-                             scale, buf, true, dtype, stream);
+                             scale, 1, buf, true, dtype, stream);
 }
 
 int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t num_problems, const void* x,
                             const int32_t* s_start, const int32_t* s_end, int32_t num_segments,
                             int64_t num_tokens, int32_t h_in, int32_t r, int64_t layer_idx, float scale,
-                            void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
+                            int32_t accumulate, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
+  if (accumulate != 0 && accumulate != 1)
+    return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (num_problems < 1 || num_problems > kMaxShrinkGroup)
     return fail(LORAX_EINVAL, "num_problems=%d (1 to %d per call)", num_problems, kMaxShrinkGroup);
   if (problems == nullptr) return fail(LORAX_EINVAL, "null pointer argument (problems)");
@@ -302,8 +308,13 @@ int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t
       if (tmp_bytes < LORAX_SHRINK_TMP_BYTES)
         return fail(LORAX_ETMPSIZE, "CHECK_GE(tmp.size(0), 8 * 1024 * 1024) failed. %lld vs %d", (long long)tmp_bytes,
                     LORAX_SHRINK_TMP_BYTES);
-      const int rc = lorax_sgmv_shrink(problems[i].v, x, problems[i].w_ptrs, s_start, s_end, num_segments, num_tokens,
-                                       h_in, r, LORAX_A_RH, layer_idx, scale, tmp, LORAX_SHRINK_TMP_BYTES, dtype, stream);
+      if (num_segments < 0 || num_tokens < 0)
+        return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments, (long long)num_tokens);
+      if (num_segments == 0 || num_tokens == 0) continue;
+      if (tmp == nullptr) return fail(LORAX_EINVAL, "null pointer argument (tmp)");
+      const int rc = sgmv_shrink_checked(problems[i].v, x, problems[i].w_ptrs, s_start, s_end, num_segments, num_tokens,
+                                         h_in, r, LORAX_A_RH, layer_idx, scale, accumulate, aligned16(tmp) ? tmp : nullptr,
+                                         false, dtype, stream);
       if (rc != LORAX_OK) return rc;
     }
     return LORAX_OK;
@@ -335,6 +346,7 @@ int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t
   a.layer_idx = layer_idx;
   a.dtype = dtype;
   a.scale = scale;
+  a.accumulate = accumulate;
   if (aligned16(tmp)) {  // fp32 partial tiles of a launch that splits K
     a.partials = static_cast<float*>(tmp);
     a.partial_bytes = static_cast<size_t>(tmp_bytes);

@@ -69,6 +69,20 @@ __device__ __forceinline__ void accumulate4(typename D::E* p, f32x4 delta) {
   *reinterpret_cast<vec4*>(p) = y;
 }
 
+// The same for a destination that is overwritten: the old value counts as zero.
+template <typename D>
+__device__ __forceinline__ void overwrite4(typename D::E* p, f32x4 delta) {
+  typedef typename D::E vec4 __attribute__((ext_vector_type(4)));
+  vec4 y;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) y[i] = from_f32<D>(delta[i]);
+  *reinterpret_cast<vec4*>(p) = y;
+}
+template <typename D>
+__device__ __forceinline__ void update4(bool add, typename D::E* p, f32x4 delta) {
+  if (add) accumulate4<D>(p, delta); else overwrite4<D>(p, delta);
+}
+
 // All tensors and weight stacks live in device (global) memory.  Weight addresses arrive as
 // integers, which the compiler can only treat as generic pointers (flat_load); the explicit
 // address space turns every 16-byte access into global_load/global_store_dwordx4.

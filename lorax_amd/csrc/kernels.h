@@ -88,7 +88,7 @@ struct SgmvArgs {
   int dtype;
   ShrinkGroup group;  // shrink of several projections: count > 1, d_out = count * rank; else unused
   float scale;     // shrink: factor applied to the fp32 sums before rounding (1 in the reference's calls)
-  int accumulate;  // expand: 1 = add to y (the reference's only mode), 0 = overwrite the rows of the segments
+  int accumulate;  // 1 = add to the destination (the reference's only mode), 0 = overwrite the rows of the segments
   // scratch of the shrink's split-K (the caller's tmp, or the library's static array): fp32 partial tiles and one
   // arrival counter per row tile; null = no scratch, the launch does not split K across workgroups
   float* partials;

@@ -25,7 +25,7 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in,
     int64_t layer_idx, int ksplit, float* __restrict__ partials,
-    uint32_t* __restrict__ counters, int num_counters, int rotate_k, float scale) {
+    uint32_t* __restrict__ counters, int num_counters, int rotate_k, float scale, int accumulate_into_v) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   constexpr int R = NB * 16;
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
           const int n = nb * 16 + 4 * (ln >> 4);
           if (row < rt.row_end) {
             if (ksplit == 1) {
-              accumulate4<D>(V + static_cast<int64_t>(row) * R + n, s * scale);
+              update4<D>(accumulate_into_v != 0, V + static_cast<int64_t>(row) * R + n, s * scale);
             } else {
               float* pp = partials + (static_cast<int64_t>(kc) * num_tokens + row) * R + n;
               *reinterpret_cast<f32x4*>(pp) = s;
@@ -187,7 +187,7 @@ __global__ __launch_bounds__(WAVES * kWave) void sgmv_shrink_rh_kernel(
             const float* pp = partials + (static_cast<int64_t>(q) * num_tokens + row) * R + n;
             s += *reinterpret_cast<const f32x4*>(pp);
           }
-          accumulate4<D>(V + static_cast<int64_t>(row) * R + n, s * scale);
+          update4<D>(accumulate_into_v != 0, V + static_cast<int64_t>(row) * R + n, s * scale);
         }
         if (tid == 0) atomicExch(&counters[tile], 0u);
       }
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void sgmv_shrink_hr_kernel(
     typename D::E* __restrict__ V, const typename D::E* __restrict__ X,
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int r,
-    int64_t layer_idx, float scale) {
+    int64_t layer_idx, float scale, int accumulate_into_v) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   constexpr int THREADS = 256;
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(256) void sgmv_shrink_hr_kernel(
         const int row = rt.row0 + tid / 8;
         if (row < rt.row_end) {
           E* vp = V + static_cast<int64_t>(row) * r + n0 + (tid % 8);
-          *vp = accumulate<D>(*vp, s * scale);
+          *vp = accumulate<D>(accumulate_into_v != 0 ? *vp : static_cast<E>(0.f), s * scale);
         }
       }
       __syncthreads();
@@ -323,7 +323,8 @@ static hipError_t launch_rh_w(const SgmvArgs& a, int ksplit, hipStream_t stream)
                      stream, static_cast<typename D::E*>(a.y),
                      static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end,
                      a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, ksplit,
-                     a.partials, a.counters, static_cast<int>(a.num_counters), tuning().shrink_no_rotate ? 0 : 1, a.scale);
+                     a.partials, a.counters, static_cast<int>(a.num_counters), tuning().shrink_no_rotate ? 0 : 1, a.scale,
+                     a.accumulate);
   return hipGetLastError();
 }
 
@@ -357,7 +358,7 @@ static hipError_t launch_shrink_dtype(const SgmvArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL((sgmv_shrink_hr_kernel<D, RT>), grid, dim3(256), 0, stream,
                        static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x),
                        a.w_ptrs, a.s_start, a.s_end, a.num_segments,
-                       static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, a.scale);
+                       static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.layer_idx, a.scale, a.accumulate);
     return hipGetLastError();
   }
   if (a.d_out % 16 != 0) return hipErrorInvalidValue;  // the register-operand kernel works in 16-column blocks

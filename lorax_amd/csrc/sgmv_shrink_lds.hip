@@ -58,7 +58,7 @@ template <typename D, int NB, int MBLK, bool KSPLIT>
 __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     const ShrinkGroup grp, const typename D::E* __restrict__ X, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int64_t layer_idx,
-    int stages, float scale) {
+    int stages, float scale, int accumulate_into_v) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   // The A tile stacks the A matrices of grp.count projections of rank r: row p * r + i is row i of
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
       const int proj = col / r;
       if (row < rt.row_end && proj < grp.count) {
         E* Vp = static_cast<E*>(proj == 0 ? grp.v[0] : (proj == 1 ? grp.v[1] : (proj == 2 ? grp.v[2] : grp.v[3])));
-        accumulate4<D>(Vp + static_cast<int64_t>(row) * r + (col - proj * r), sum * scale);
+        update4<D>(accumulate_into_v != 0, Vp + static_cast<int64_t>(row) * r + (col - proj * r), sum * scale);
       }
     };
     if constexpr (KSPLIT) {
@@ -266,7 +266,7 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, grp, static_cast<const typename D::E*>(a.x),
                      a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages,
-                     a.scale);
+                     a.scale, a.accumulate);
   return hipGetLastError();
 }
 

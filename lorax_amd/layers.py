@@ -13,6 +13,8 @@ Deliberate differences from the reference:
     through the kernels' column window instead of through a zero-filled staging tensor
     and a second pass (:109-112,166-167).  Every token belongs to at most one rank
     group, so both orders round identically;
+  * in prefill the shrink overwrites the rows of the segments in v, so v is not zero-filled first
+    (utils/punica.py:176-178 allocates zeros); the expand reads no other rows;
   * in decode, the projections of one layer that share an input (q/k/v, gate/up) go to the
     GPU as ONE shrink launch and ONE expand launch per rank (``lorax_bgmv_multi``), and the
     shrink overwrites v, so there is no zero-fill (:146).  A decode-size BGMV is shorter
@@ -118,7 +120,7 @@ class LoraLinear(nn.Module):
                         continue
                     v = lora_a_sgmv_resident(
                         input, get_shrink_scratch(input.device), rs.lora_a_t_ptr, rs.segment_starts, rs.segment_ends,
-                        self.layer_id, r,
+                        self.layer_id, r, zero_fill=tensor_parallel,
                     )
                 else:
                     v = lora_a_sgmv_cutlass(
@@ -151,7 +153,7 @@ class LoraLinear(nn.Module):
                 first = chunk[0][0]
                 vs = lora_a_sgmv_resident_multi(
                     input, get_shrink_scratch(input.device), [rs.lora_a_t_ptr for rs, _, _ in chunk],
-                    first.segment_starts, first.segment_ends, self.layer_id, r,
+                    first.segment_starts, first.segment_ends, self.layer_id, r, zero_fill=False,
                 )
                 for v, (rs, start, width) in zip(vs, chunk):
                     lora_b_sgmv_cutlass_slice(

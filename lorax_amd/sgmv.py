@@ -153,11 +153,15 @@ def lora_a_sgmv_resident(
     s_end: torch.IntTensor,
     layer_idx: int,
     lora_rank: int,
+    zero_fill: bool = True,
 ) -> torch.Tensor:
     """As lora_a_sgmv_cutlass, reading the [L, r, h_in] stacks of the decode path (weights_a_t) whatever
-    the rank.  `tmp` is get_shrink_scratch(device) or the 8 MiB buffer of get_tmp_tensor."""
-    v = torch.zeros((x.size(0), lora_rank), dtype=x.dtype, device=x.device)
-    _native_module().sgmv_shrink_multi([v], x, [wa_t_ptr], s_start, s_end, tmp, layer_idx)
+    the rank.  `tmp` is get_shrink_scratch(device) or the 8 MiB buffer of get_tmp_tensor.
+    zero_fill=False skips the zero-fill launch: the kernel overwrites the rows of the segments and the rows
+    outside every segment hold garbage - fine for a v that only goes to the expand of the same segments."""
+    alloc = torch.zeros if zero_fill else torch.empty
+    v = alloc((x.size(0), lora_rank), dtype=x.dtype, device=x.device)
+    _native_module().sgmv_shrink_multi([v], x, [wa_t_ptr], s_start, s_end, tmp, layer_idx, 1.0, zero_fill)
     return v
 
 
@@ -169,13 +173,15 @@ def lora_a_sgmv_resident_multi(
     s_end: torch.IntTensor,
     layer_idx: int,
     lora_rank: int,
+    zero_fill: bool = True,
 ) -> List[torch.Tensor]:
     """lora_a_sgmv_resident for up to 4 projections that share x, the segments and the rank (q/k/v, gate/up):
     one v per pointer table.  One launch that reads x once when the summed rank is at most 128 and h_in a
     multiple of 128; the reference issues one shrink per projection (layers.py:121-133)."""
-    flat = torch.zeros((len(wa_t_ptrs), x.size(0), lora_rank), dtype=x.dtype, device=x.device)
+    alloc = torch.zeros if zero_fill else torch.empty
+    flat = alloc((len(wa_t_ptrs), x.size(0), lora_rank), dtype=x.dtype, device=x.device)
     vs = list(flat.unbind(0))
-    _native_module().sgmv_shrink_multi(vs, x, list(wa_t_ptrs), s_start, s_end, tmp, layer_idx)
+    _native_module().sgmv_shrink_multi(vs, x, list(wa_t_ptrs), s_start, s_end, tmp, layer_idx, 1.0, zero_fill)
     return vs
 
 

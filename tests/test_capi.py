@@ -79,18 +79,20 @@ def test_sgmv_shrink_multi_validation():
     big = 8 * 1024 * 1024
     one = (_native.SgmvShrinkProblem * 1)(_native.SgmvShrinkProblem(P, P))
     two = (_native.SgmvShrinkProblem * 2)(_native.SgmvShrinkProblem(P, P), _native.SgmvShrinkProblem(P, P))
-    assert f(two, 0, P, P, P, 2, 1000, 4096, 16, 0, 1.0, P, big, 1, None) == EINVAL and "num_problems" in _err()
-    assert f(two, 5, P, P, P, 2, 1000, 4096, 16, 0, 1.0, P, big, 1, None) == EINVAL
-    assert f(None, 2, P, P, P, 2, 1000, 4096, 16, 0, 1.0, P, big, 1, None) == EINVAL
+    assert f(two, 0, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, 1, None) == EINVAL and "num_problems" in _err()
+    assert f(two, 5, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, 1, None) == EINVAL
+    assert f(None, 2, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, 1, None) == EINVAL
     # stacked launch (2 x 64 <= 128, h_in a multiple of 128, more than 512 rows): its own checks
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, P, big - 1, 1, None) == ETMPSIZE
-    assert f(two, 2, P, P, P, 0, 1000, 4096, 64, 0, 1.0, P, big, 1, None) == OK  # no segments
-    assert f(two, 2, P, P, None, 2, 1000, 4096, 64, 0, 1.0, P, big, 1, None) == EINVAL and "null" in _err()
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, -1, 1.0, P, big, 1, None) == EINVAL
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 1, P, big - 1, 1, None) == ETMPSIZE
+    assert f(two, 2, P, P, P, 0, 1000, 4096, 64, 0, 1.0, 1, P, big, 1, None) == OK  # no segments
+    assert f(two, 2, P, P, None, 2, 1000, 4096, 64, 0, 1.0, 1, P, big, 1, None) == EINVAL and "null" in _err()
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, -1, 1.0, 1, P, big, 1, None) == EINVAL
     # one launch per projection (summed rank 192; or a single projection): lorax_sgmv_shrink's checks
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 96, 0, 1.0, P, big - 1, 1, None) == ETMPSIZE
-    assert f(one, 1, P, P, P, 2, 1000, 4100, 16, 0, 1.0, P, big, 1, None) == ENOKERNEL
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 12, 0, 1.0, P, big, 1, None) == ENOKERNEL
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 96, 0, 1.0, 1, P, big - 1, 1, None) == ETMPSIZE
+    assert f(one, 1, P, P, P, 2, 1000, 4100, 16, 0, 1.0, 1, P, big, 1, None) == ENOKERNEL
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 12, 0, 1.0, 1, P, big, 1, None) == ENOKERNEL
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 2, P, big, 1, None) == EINVAL and "accumulate" in _err()
+    assert f(two, 2, P, P, P, 0, 1000, 4096, 64, 0, 1.0, 0, P, 4 * big, 1, None) == OK  # a larger scratch is accepted
 
 
 def test_sgmv_expand_validation():

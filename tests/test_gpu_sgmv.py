@@ -8,7 +8,7 @@ from pathlib import Path
 import pytest
 import torch
 
-from lorax_amd import sgmv
+from lorax_amd import _native, sgmv
 from oracle import lora_oracle as O
 from tests.helpers import assert_close, ptr_table, randn, stored_sgmv_a
 
@@ -411,10 +411,17 @@ def test_sgmv_shrink_multi(dtype, count, r, h_in, lens):
     tables = [ptr_table(ws, DEV) for ws in stacks]
     vs = sgmv.lora_a_sgmv_resident_multi(x, tmp, tables, s_start, s_end, layer, r)
     singles = [sgmv.lora_a_sgmv_resident(x, tmp, t, s_start, s_end, layer, r) for t in tables]
+    # overwrite mode: same values in the rows of the segments whatever v held, other rows untouched
+    dirty = [torch.full((T, r), 7.0, dtype=dtype, device=DEV) for _ in tables]
+    _native.sgmv_shrink_multi(dirty, x, tables, s_start, s_end, sgmv.get_shrink_scratch(torch.device(DEV)), layer, 1.0,
+                              accumulate=False)
     torch.cuda.synchronize()
     covered = torch.zeros(T, dtype=torch.bool)
     for s, e in zip(starts, ends):
         covered[s:e] = True
+    for p in range(count):
+        assert torch.equal(dirty[p].cpu()[covered], vs[p].cpu()[covered])
+        assert torch.all(dirty[p].cpu()[~covered] == 7.0)
     for p in range(count):
         v_ref = torch.zeros((T, r), dtype=dtype)
         for i, (s, e) in enumerate(zip(starts, ends)):
