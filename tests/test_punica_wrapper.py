@@ -40,7 +40,7 @@ def test_update_metadata_shifts_adapter_indices_by_the_base_model_slot():
     starts, lengths, idx, batches, longest = wrapper.prefill_metadata
     assert (starts.tolist(), lengths.tolist(), idx.tolist(), batches, longest) == ([0, 2, 4, 5], [2, 2, 1, 1],
                                                                                    [-1, 0, 2, -1], 4, 2)
-    s, e = wrapper._bounds
+    s, e = wrapper._kernel_bounds
     assert s.tolist() == [0, 2, 4, 5] and e.tolist() == [0, 4, 5, 5]
     wrapper.update_metadata(make_meta([2, 0, 1], torch.device("cpu")), prefill=False)
     assert not wrapper.is_prefill and wrapper.token_lora_indices.tolist() == [1, -1, 0]
@@ -76,3 +76,27 @@ def test_stack_table_addresses_every_entry():
     assert table.dtype == torch.int64
     assert table.tolist() == [w.data_ptr() + i * 8 * 32 * 2 for i in range(5)]
     assert ops.stack_table(w) is table  # cached per weight tensor
+
+
+def test_run_table_taken_from_the_batch_equals_the_one_computed_from_the_tokens():
+    """update_metadata reuses adapter_segments / segment_indices when the metadata carries them; a metadata object
+    with only per-token indices goes through _update_prefill_metada.  Both give the same state."""
+    from types import SimpleNamespace
+
+    tokens = [2, 2, 0, 0, 0, 5, 2, 2, 0]
+    full = make_meta(tokens, torch.device("cpu"))
+    bare = SimpleNamespace(adapter_indices=full.adapter_indices)
+    a = PunicaWrapper(max_num_batched_tokens=16, max_batches=8, device="cpu", enabled=True)
+    b = PunicaWrapper(max_num_batched_tokens=16, max_batches=8, device="cpu", enabled=True)
+    a.update_metadata(full, prefill=True)
+    b.update_metadata(bare, prefill=True)
+    for x, y in zip(a.prefill_metadata, b.prefill_metadata):
+        assert (x.tolist() == y.tolist()) if isinstance(x, torch.Tensor) else x == y
+    assert a.prefill_metadata[3:] == (5, 3) and a.no_lora == b.no_lora is False
+    assert [t.tolist() for t in a._kernel_bounds] == [t.tolist() for t in b._kernel_bounds] == [[0, 2, 5, 6, 8],
+                                                                                               [2, 2, 6, 8, 8]]
+    # a batch of base-model tokens only: nothing is routed
+    for w, m in ((a, make_meta([0, 0, 0], torch.device("cpu"))),
+                 (b, SimpleNamespace(adapter_indices=torch.tensor([0, 0, 0])))):
+        w.update_metadata(m, prefill=True)
+        assert w.no_lora and w.batch_size == 1
