@@ -114,6 +114,7 @@ struct Tuning {
   int bgmv_no_runs;   // LORAX_BGMV_NO_RUNS: number workgroups problem by problem
   int bgmv_no_balance;  // LORAX_BGMV_NO_BALANCE: plain workgroup numbering in the single-launch BGMV
   int shrink_rows_max;  // LORAX_SHRINK_ROWS_MAX: largest token count served by the streaming SGMV shrink (-1 = never)
+  int shrink_rows;      // LORAX_SHRINK_ROWS: rows per tile of the LDS-staged SGMV shrink (below its buffers' height)
 };
 const Tuning& tuning();
 

@@ -58,7 +58,7 @@ template <typename D, int NB, int MBLK, bool KSPLIT>
 __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     const ShrinkGroup grp, const typename D::E* __restrict__ X, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int64_t layer_idx,
-    int stages, float scale, int accumulate_into_v) {
+    int stages, float scale, int accumulate_into_v, int rows_per_tile) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   // The A tile stacks the A matrices of grp.count projections of rank r: row p * r + i is row i of
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
   constexpr int WN = KSPLIT ? 1 : ((NB % 2 == 0) ? 2 : 1);
   constexpr int WM = KSPLIT ? 1 : 4 / WN;
   static_assert(MBLK % WM == 0, "row blocks must divide among the waves");
-  static_assert(!KSPLIT || 4 * MBLK * NB * 1024 <= 2 * kStageBytes, "partial sums must fit in two stage buffers");
+  // KSPLIT: the partial sums (4 * MBLK * NB KB) go where the stage buffers are; the launcher sizes the LDS for it
   constexpr int MPW = MBLK / WM;  // row blocks per wave
   constexpr int NPW = NB / WN;    // rank blocks per wave
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -98,7 +98,8 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
 
   for (int tile = vb.x;; tile += gridDim.x) {
     RowTile rt;
-    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, ROWS, tile, rt)) break;
+    // tiles may be lower than the ROWS the buffers hold: rows past a tile's end re-read its last row
+    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const E* A[kMaxShrinkGroup];
 #pragma unroll
     for (int p = 0; p < kMaxShrinkGroup; ++p)
@@ -232,7 +233,20 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
 template <typename D, int NB, int MBLK, bool KSPLIT>
 static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   constexpr int kStageBytes = (MBLK + NB) * 16 * kLdsRowBytes;
-  const int64_t tiles = (a.num_tokens + MBLK * 16 - 1) / (MBLK * 16) + a.num_segments;
+  constexpr int kRedBytes = KSPLIT ? 4 * MBLK * NB * 1024 : 0;  // partial sums of the four waves at the end of a tile
+  static_assert(kRedBytes <= kLdsMaxBytes, "partial sums must fit in LDS");
+  // Tile height: a launch streams at the rate of the CUs that have a workgroup, so when the full-height tiles
+  // are fewer than the 256 CUs the tiles are lowered (in steps of 16 rows) until they are about as many.  The
+  // host knows the rows and the number of segments, not their lengths: ceil(T / M) + segments bounds the count.
+  int rows_per_tile = MBLK * 16;
+  if (tuning().shrink_rows <= 0) {
+    while (rows_per_tile > 16 &&
+           (a.num_tokens + rows_per_tile - 17) / (rows_per_tile - 16) + a.num_segments <= 256)
+      rows_per_tile -= 16;
+  } else if (tuning().shrink_rows < rows_per_tile) {
+    rows_per_tile = (tuning().shrink_rows + 15) / 16 * 16;
+  }
+  const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
   // Stage buffers: all of a CU's LDS when there is at most one workgroup per CU; a third of it when the
   // tiles make one to three rounds over the CUs (more resident workgroups even out the last round);
   // half of it for long launches.  2 to 8 stages.
@@ -242,7 +256,8 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   stages = stages < 2 ? 2 : (stages > kLdsMaxStages ? kLdsMaxStages : stages);
   static_assert(2 * kStageBytes <= kLdsMaxBytes, "two stages must fit in LDS");
   while (stages * kStageBytes > kLdsMaxBytes) --stages;
-  const int lds_bytes = stages * kStageBytes;
+  int lds_bytes = stages * kStageBytes;
+  if (lds_bytes < kRedBytes) lds_bytes = kRedBytes;
   auto kernel = sgmv_shrink_lds_kernel<D, NB, MBLK, KSPLIT>;
   // Raising the dynamic LDS limit is needed once per kernel and device.
   static bool configured[64] = {};
@@ -266,7 +281,7 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, grp, static_cast<const typename D::E*>(a.x),
                      a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages,
-                     a.scale, a.accumulate);
+                     a.scale, a.accumulate, rows_per_tile);
   return hipGetLastError();
 }
 
@@ -282,6 +297,8 @@ static hipError_t launch_lds_nb(const SgmvArgs& a, hipStream_t stream) {
   if (tuning().shrink_mb > 0) mblk = tuning().shrink_mb;
   const bool ksplit = tuning().shrink_lds != 2;
   if (mblk >= 4) {
+    // every staged byte read from LDS once (k slices per wave) up to rank 64; above, the waves split the output
+    // blocks instead (k slices at rank 128 need 128 accumulator registers per lane and measured no faster)
     if constexpr (NB <= 4) {
       if (ksplit) return launch_lds_m<D, NB, 4, true>(a, stream);
     }
