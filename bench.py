@@ -127,6 +127,10 @@ class Plan:
                     decode[r].append((rd, off, size))
             # as lorax_amd.layers: projections of one rank and the same segment tables shrink in one launch
             for (r, _), same in prefill.items():
+                if fuse_small_ranks and _native.sgmv_lora_fits(r, group.h_in, T):
+                    for i in range(0, len(same), _native.MAX_FUSED_BGMV_PROBLEMS):
+                        self._add_sgmv_fused(x, y, group.h_in, r, same[i:i + _native.MAX_FUSED_BGMV_PROBLEMS])
+                    continue
                 step = max(1, min(_native.MAX_SGMV_SHRINK_PROBLEMS, 128 // r))
                 for i in range(0, len(same), step):
                     self._add_sgmv_group(x, y, group.h_in, r, same[i:i + step])
@@ -224,6 +228,26 @@ class Plan:
 
             self.calls.append(("sgmv_expand", expand, rows * r * e + uniq * r * size * e + 2 * rows * size * e,
                                2 * rows * r * size, rows * r * e + rows * r * size * e + 2 * rows * size * e))
+
+    def _add_sgmv_fused(self, x, y, h_in, r, jobs):
+        """Shrink and expand of up to four projections of a short prefill batch in one launch; v stays on chip."""
+        from lorax_amd import _native
+
+        e = 2
+        first = jobs[0][0]
+        starts, ends = first.segment_starts, first.segment_ends
+        lens = (ends - starts).clamp(min=0)
+        rows = int(lens.sum().item())
+        problems = [(y, rd.lora_a_t_ptr, rd.lora_b_t_ptr, off, size) for rd, off, size in jobs]
+        nbytes = gather = rows * h_in * e
+        flops = 0
+        for rd, _, size in jobs:
+            uniq = len(set(rd.lora_a_t_ptr[lens > 0].tolist()))
+            nbytes += uniq * r * (h_in + size) * e + 2 * rows * size * e
+            gather += rows * r * (h_in + size) * e + 2 * rows * size * e
+            flops += 2 * rows * r * (h_in + size)
+        self.calls.append(("sgmv_lora", lambda layer: _native.sgmv_lora_multi(problems, x, starts, ends, r, layer),
+                           nbytes, flops, gather))
 
     def _add_bgmv_reference(self, x, y, off, size, h_in, r, rd):
         import torch

@@ -215,6 +215,30 @@ int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t
                             int32_t accumulate, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
 
 /*
+ * Shrink and expand of a SHORT prefill batch in one launch, for up to 4 projections that share x and the
+ * segment tables:
+ *   y_p[s:e, y_offset_p : y_offset_p + h_out_p] += dtype(scale * dtype(x[s:e] @ A_p,i^T) @ B_p,i^T)   per segment i
+ * with A_p,i = a_ptrs_p[i] ([num_layers, r, h_in] stack) and B_p,i = b_ptrs_p[i] ([num_layers, h_out, r] stack).
+ * No counterpart in the reference: it is the sequence zero-fill, sgmv_shrink, sgmv_cutlass of
+ * lorax_server/utils/layers.py:114-142 (punica.py:170-196) without the intermediate tensor and two of the three
+ * launches, for batches that are bound by launches rather than bytes.  The intermediate x @ A^T is rounded to
+ * dtype exactly where the two-call sequence rounds it when it stores v.  r must be 8 or 16 and num_tokens at
+ * most 512; empty and negative segments are skipped without reading their table entries' stacks.
+ */
+typedef struct lorax_sgmv_lora_problem {
+  void* y;                /* [num_tokens, y_stride]                                  */
+  const int64_t* a_ptrs;  /* [num_segments] device addresses of [L, r, h_in] stacks  */
+  const int64_t* b_ptrs;  /* [num_segments] device addresses of [L, h_out, r] stacks */
+  int64_t y_offset;
+  int64_t y_stride;
+  int32_t h_out;
+} lorax_sgmv_lora_problem_t;
+
+int lorax_sgmv_lora_multi(const lorax_sgmv_lora_problem_t* problems, int32_t num_problems, const void* x,
+                          const int32_t* s_start, const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
+                          int32_t h_in, int32_t r, int64_t layer_idx, float scale, int32_t dtype, void* stream);
+
+/*
  * SGMV expand.  Replaces the expand direction of sgmv_cutlass (punica_ops.cc:338-367,
  * sgmv/sgmv_cutlass.cuh:86-131).
  *

@@ -48,6 +48,13 @@ class SgmvShrinkProblem(ctypes.Structure):
     _fields_ = [("v", _c.c_void_p), ("w_ptrs", _c.c_void_p)]
 
 
+class SgmvLoraProblem(ctypes.Structure):
+    """lorax_sgmv_lora_problem_t of include/lorax_hip.h."""
+
+    _fields_ = [("y", _c.c_void_p), ("a_ptrs", _c.c_void_p), ("b_ptrs", _c.c_void_p), ("y_offset", _c.c_int64),
+                ("y_stride", _c.c_int64), ("h_out", _c.c_int32)]
+
+
 class AdapterEntry(ctypes.Structure):
     """lorax_adapter_entry_t of include/lorax_hip.h."""
 
@@ -99,6 +106,11 @@ _SIGNATURES = {
         [_c.POINTER(SgmvShrinkProblem), _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
          _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_int32, _c.c_void_p, _c.c_int64, _c.c_int32,
          _c.c_void_p],
+    ),
+    "lorax_sgmv_lora_multi": (
+        _c.c_int,
+        [_c.POINTER(SgmvLoraProblem), _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
+         _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_int32, _c.c_void_p],
     ),
     "lorax_sgmv_expand": (
         _c.c_int,
@@ -448,6 +460,48 @@ def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: floa
             ys[0].size(1), int(layer_idx), float(scale), 1 if accumulate else 0, tmp.data_ptr(),
             tmp.numel() * tmp.element_size(), _dtype_code(x), _stream(x),
         )
+    if rc != 0:
+        _raise_last(rc)
+
+
+SGMV_LORA_MAX_TOKENS = 512
+
+
+def sgmv_lora_fits(rank: int, h_in: int, num_tokens: int) -> bool:
+    """True where the single-launch prefill update (lorax_sgmv_lora_multi) applies and pays: rank 8 or 16 with a
+    small A slab, and a batch short enough to be bound by launches."""
+    return rank in FUSED_BGMV_RANKS and rank * h_in * 2 <= 128 * 1024 and num_tokens <= SGMV_LORA_MAX_TOKENS
+
+
+def sgmv_lora_multi(problems, x, s_start, s_end, rank, layer_idx, scale: float = 1.0) -> None:
+    """lorax_sgmv_lora_multi: `problems` is a list of up to 4 tuples (y, a_t_ptr, b_t_ptr, y_offset, y_slice_size)
+    whose projections share x and the segment tables; y[s:e, window] += (x[s:e] @ A_i^T) @ B_i^T per segment,
+    rank 8 or 16, at most 512 rows, in one launch."""
+    if not 1 <= len(problems) <= MAX_FUSED_BGMV_PROBLEMS:
+        raise RuntimeError(f"between 1 and {MAX_FUSED_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
+    _check_input(x, "x", 2)
+    _check_input(s_start, "s_start", 1)
+    _check_input(s_end, "s_end", 1)
+    if s_start.dtype != torch.int32 or s_end.dtype != torch.int32 or s_start.size(0) != s_end.size(0):
+        raise RuntimeError("s_start and s_end must be int32 tensors of one length")
+    arr = (SgmvLoraProblem * len(problems))()
+    for i, (y, a_ptr, b_ptr, y_offset, y_slice_size) in enumerate(problems):
+        _check_input(y, "y", 2)
+        _check_input(a_ptr, "a_ptr", 1)
+        _check_input(b_ptr, "b_ptr", 1)
+        _check_same(y, x, a_ptr, b_ptr, s_start, s_end)
+        if a_ptr.dtype != torch.int64 or b_ptr.dtype != torch.int64:
+            raise RuntimeError("a_ptr and b_ptr must be int64 tensors")
+        if a_ptr.size(0) != s_start.size(0) or b_ptr.size(0) != s_start.size(0):
+            raise RuntimeError("a_ptr and b_ptr must have one entry per segment")
+        if y.size(0) != x.size(0):
+            raise RuntimeError(f"CHECK_EQ(y.size(0), x.size(0)) failed. {y.size(0)} vs {x.size(0)}")
+        h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
+        arr[i] = SgmvLoraProblem(y.data_ptr(), a_ptr.data_ptr(), b_ptr.data_ptr(), int(y_offset), y.size(1), h_out)
+    with torch.cuda.device(x.device):
+        rc = lib().lorax_sgmv_lora_multi(arr, len(problems), x.data_ptr(), s_start.data_ptr(), s_end.data_ptr(),
+                                         s_start.size(0), x.size(0), x.size(1), int(rank), int(layer_idx),
+                                         float(scale), _dtype_code(x), _stream(x))
     if rc != 0:
         _raise_last(rc)
 

@@ -208,13 +208,14 @@ __global__ __launch_bounds__(kBgmvThreads) void sgmv_shrink_rows_kernel(
   const int v = static_cast<int>(xcd_virtual_id());
   const int chunk = v / subs;
   const int row0 = (v % subs) * RS;
+  const int64_t pre = preload_segment_entry(W, num_segments);
   RowTile rt;
   if (!find_row_tile(s_start, s_end, num_segments, num_tokens, kGroup, chunk, rt)) return;
   const int n = rt.row_end - rt.row0;
   int toks[kGroup];
 #pragma unroll
   for (int g = 0; g < kGroup; ++g) toks[g] = rt.row0 + min(g, n - 1);
-  const E* A = reinterpret_cast<const E*>(W[rt.seg]) + (layer_idx * r + row0) * static_cast<int64_t>(h_in);
+  const E* A = reinterpret_cast<const E*>(segment_entry(pre, W, rt.seg)) + (layer_idx * r + row0) * static_cast<int64_t>(h_in);
   switch (n) {
     case 1:
       bgmv_shrink_body<D, RS, 1>(V, X, A, toks, h_in, row0, 0, r, scale, acc_v, red);
@@ -690,6 +691,82 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch
   else
     bgmv_lora_tokens<D, R, U, NBLK, VEC4>(n, Y, X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset, P.y_stride,
                                           scale, red, vsh);
+}
+
+// ---------------------------------------------------------------------------------
+// Shrink and expand of a SHORT prefill batch in one launch: the body above with the token chunks cut from the
+// segments (4 consecutive rows of one segment) instead of gathered by adapter.  A prefill batch of a few dozen
+// rows is bound by launches - zero-fill, shrink and expand take about 4 us each for a megabyte of traffic - so
+// the whole update of up to four projections that share x goes out as one.
+// ---------------------------------------------------------------------------------
+template <typename D, int R, int U, int NBLK, bool VEC4>
+__global__ __launch_bounds__(kBgmvThreads) void sgmv_lora_rows_kernel(
+    const SgmvLoraBatch batch, const typename D::E* __restrict__ X, const int32_t* __restrict__ s_start,
+    const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int64_t layer_idx, float scale) {
+  using E = typename D::E;
+  __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<R * kGroup>::value];
+  __shared__ __attribute__((aligned(16))) E vsh[R * kGroup];
+  const VirtualBlock vb = xcd_virtual_block();  // x: column slice, y: row chunk, z: projection
+  const SgmvLoraProblem& P = batch.p[vb.z];
+  const int h_out = P.h_out;
+  constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
+  const int col0 = vb.x * cols_per_wg;
+  if (col0 >= h_out) return;
+  const int col_end = min(col0 + cols_per_wg, h_out);
+  const int64_t pre_a = preload_segment_entry(P.a_ptrs, num_segments);
+  const int64_t pre_b = preload_segment_entry(P.b_ptrs, num_segments);
+  RowTile rt;
+  if (!find_row_tile(s_start, s_end, num_segments, num_tokens, kGroup, vb.y, rt)) return;
+  const int n = rt.row_end - rt.row0;
+  int toks[kGroup];
+#pragma unroll
+  for (int g = 0; g < kGroup; ++g) toks[g] = rt.row0 + min(g, n - 1);
+  const E* A = reinterpret_cast<const E*>(segment_entry(pre_a, P.a_ptrs, rt.seg)) + layer_idx * R * static_cast<int64_t>(h_in);
+  const E* B = reinterpret_cast<const E*>(segment_entry(pre_b, P.b_ptrs, rt.seg)) + layer_idx * h_out * static_cast<int64_t>(R);
+  bgmv_lora_tokens<D, R, U, NBLK, VEC4>(n, static_cast<E*>(P.y), X, A, B, toks, h_in, h_out, col0, col_end, P.y_offset,
+                                        P.y_stride, scale, red, vsh);
+}
+
+template <typename D, int R, int NBLK>
+static hipError_t launch_sgmv_lora_blk(const SgmvLoraArgs& a, hipStream_t stream) {
+  constexpr int U = 4;
+  constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
+  int wide = 0;
+  bool vec4 = true;  // 8-byte y accesses need every problem's rows 8-byte aligned and no ragged last column group
+  for (int i = 0; i < a.count; ++i) {
+    const SgmvLoraProblem& p = a.batch.p[i];
+    wide = p.h_out > wide ? p.h_out : wide;
+    vec4 = vec4 && p.h_out % 4 == 0 && p.y_stride % 4 == 0 && p.y_offset % 4 == 0 &&
+           reinterpret_cast<uintptr_t>(p.y) % 8 == 0;
+  }
+  const int64_t chunks = (a.num_tokens + kGroup - 1) / kGroup + a.num_segments;  // upper bound
+  const dim3 grid((wide + cols_per_wg - 1) / cols_per_wg, static_cast<unsigned>(chunks), a.count);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(kBgmvThreads), 0, stream, a.batch, static_cast<const typename D::E*>(a.x),
+                       a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.h_in, a.layer_idx, a.scale);
+  };
+  if (vec4) launch(sgmv_lora_rows_kernel<D, R, U, NBLK, true>);
+  else launch(sgmv_lora_rows_kernel<D, R, U, NBLK, false>);
+  return hipGetLastError();
+}
+
+template <typename D, int R>
+static hipError_t launch_sgmv_lora_r(const SgmvLoraArgs& a, hipStream_t stream) {
+  // column slices as wide as the launch affords, as in launch_lora_r: every slice repeats the shrink
+  constexpr int cols4 = (kBgmvThreads / (R / 8)) * 4 * 4;
+  const int64_t chunks = (a.num_tokens + kGroup - 1) / kGroup;
+  int64_t wgs4 = 0;
+  for (int i = 0; i < a.count; ++i) wgs4 += chunks * ((a.batch.p[i].h_out + cols4 - 1) / cols4);
+  if (wgs4 >= 200) return launch_sgmv_lora_blk<D, R, 4>(a, stream);
+  if (wgs4 >= 100) return launch_sgmv_lora_blk<D, R, 2>(a, stream);
+  return launch_sgmv_lora_blk<D, R, 1>(a, stream);
+}
+
+// y[s:e, window] += T(scale * T(x[s:e] @ A_i^T) @ B_i^T) per segment, ranks 8 and 16, short batches.
+hipError_t launch_sgmv_lora_rows(const SgmvLoraArgs& a, hipStream_t stream) {
+  if (a.dtype == LORAX_F16)
+    return a.rank == 8 ? launch_sgmv_lora_r<F16, 8>(a, stream) : launch_sgmv_lora_r<F16, 16>(a, stream);
+  return a.rank == 8 ? launch_sgmv_lora_r<BF16, 8>(a, stream) : launch_sgmv_lora_r<BF16, 16>(a, stream);
 }
 
 // ---------------------------------------------------------------------------------

@@ -451,6 +451,50 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
   return LORAX_OK;
 }
 
+int lorax_sgmv_lora_multi(const lorax_sgmv_lora_problem_t* problems, int32_t num_problems, const void* x,
+                          const int32_t* s_start, const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
+                          int32_t h_in, int32_t r, int64_t layer_idx, float scale, int32_t dtype, void* stream) {
+  if (num_problems < 1 || num_problems > kMaxSgmvLoraProblems)
+    return fail(LORAX_EINVAL, "num_problems=%d (1 to %d per launch)", num_problems, kMaxSgmvLoraProblems);
+  if (num_segments < 0 || num_tokens < 0)
+    return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments, (long long)num_tokens);
+  if (num_segments == 0 || num_tokens == 0) return LORAX_OK;
+  if (problems == nullptr || s_start == nullptr || s_end == nullptr)
+    return fail(LORAX_EINVAL, "null pointer argument (problems=%p s_start=%p s_end=%p)", (const void*)problems,
+                (const void*)s_start, (const void*)s_end);
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  if ((r != 8 && r != 16) || h_in <= 0 || h_in % 8 != 0 || h_in >= 65536 || num_tokens > 512)
+    return fail(LORAX_ENOKERNEL,
+                "No suitable kernel. the single-launch prefill update covers rank 8 and 16 and up to 512 rows, "
+                "h_in=%d r=%d num_tokens=%lld", h_in, r, (long long)num_tokens);
+  SgmvLoraArgs a{};
+  a.count = num_problems;
+  a.x = x;
+  a.s_start = s_start;
+  a.s_end = s_end;
+  a.num_segments = num_segments;
+  a.num_tokens = num_tokens;
+  a.h_in = h_in;
+  a.rank = r;
+  a.layer_idx = layer_idx;
+  a.scale = scale;
+  a.dtype = dtype;
+  for (int i = 0; i < num_problems; ++i) {
+    const lorax_sgmv_lora_problem_t& q = problems[i];
+    if (int rc = check_common(q.y, x, q.a_ptrs, dtype)) return rc;
+    if (q.b_ptrs == nullptr) return fail(LORAX_EINVAL, "null pointer argument (b_ptrs)");
+    if (q.h_out <= 0 || q.h_out % 8 != 0 || q.h_out >= 65536)
+      return fail(LORAX_ENOKERNEL, "No suitable kernel. h_in=%d h_out=%d dtype=%d", h_in, q.h_out, dtype);
+    if (q.y_offset < 0 || q.y_stride < q.y_offset + q.h_out)
+      return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld do not hold h_out=%d columns", (long long)q.y_offset,
+                  (long long)q.y_stride, q.h_out);
+    a.batch.p[i] = SgmvLoraProblem{q.y, q.a_ptrs, q.b_ptrs, q.y_offset, q.y_stride, q.h_out};
+  }
+  const hipError_t e = launch_sgmv_lora_rows(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_lora launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
 size_t lorax_sgmv_tmp_size(int32_t num_problems) {
   // 3 pointers + 3 int64 leading dimensions + one (m, n, k) int32 triple per problem
   return num_problems > 0 ? static_cast<size_t>(num_problems) * (3 * 8 + 3 * 8 + 12) : 0;

@@ -97,6 +97,36 @@ struct SgmvArgs {
   size_t num_counters;
 };
 
+// Shrink and expand of a short prefill batch in one launch (bgmv.hip): up to four projections that share x and
+// the segment tables, each with its own stack tables and column window of y.
+constexpr int kMaxSgmvLoraProblems = 4;
+struct SgmvLoraProblem {
+  void* y;
+  const int64_t* a_ptrs;  // [num_segments] addresses of [L, r, h_in] stacks
+  const int64_t* b_ptrs;  // [num_segments] addresses of [L, h_out, r] stacks
+  int64_t y_offset;
+  int64_t y_stride;
+  int h_out;
+};
+struct SgmvLoraBatch {
+  SgmvLoraProblem p[kMaxSgmvLoraProblems];
+};
+struct SgmvLoraArgs {
+  SgmvLoraBatch batch;
+  int count;
+  const void* x;
+  const int32_t* s_start;
+  const int32_t* s_end;
+  int num_segments;
+  int64_t num_tokens;
+  int h_in;
+  int rank;
+  int64_t layer_idx;
+  float scale;
+  int dtype;
+};
+hipError_t launch_sgmv_lora_rows(const SgmvLoraArgs& a, hipStream_t stream);
+
 // Launch parameters that can be overridden from the environment for tuning runs, read once per process;
 // 0 (unset) = the launcher's heuristic.
 struct Tuning {

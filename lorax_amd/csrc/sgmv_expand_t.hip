@@ -80,10 +80,11 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     l_off[s] = s * 32 + (lane & 3) * 8 < r ? s * 32 + (lane & 3) * 8 : 0;
   }
 
+  const int64_t pre_w = preload_segment_entry(W, num_segments);
   for (int tile = vid % tile_slots;; tile += tile_slots) {
     RowTile rt;
     if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
-    const E* BT = reinterpret_cast<const E*>(W[rt.seg]) + layer_idx * h_out * static_cast<int64_t>(r);
+    const E* BT = reinterpret_cast<const E*>(segment_entry(pre_w, W, rt.seg)) + layer_idx * h_out * static_cast<int64_t>(r);
     const int nmb = (rt.row_end - rt.row0 + 15) / 16;
 
     for (int pp = 0; pp < panels_per_wave; ++pp) {

@@ -91,4 +91,19 @@ __device__ __forceinline__ bool find_row_tile(const int32_t* __restrict__ s_star
   return false;
 }
 
+// The stack address of a tile's segment without a memory round trip after the tile search: every lane asks for
+// the table entry of "its" segment BEFORE the search (the loads travel together with the search's own), and the
+// entry of the segment the search lands on is read from that lane afterwards.  Segments past the first 64 fall
+// back to a load.  Table entries are only read, never dereferenced, here.
+__device__ __forceinline__ int64_t preload_segment_entry(const int64_t* __restrict__ table, int num_segments) {
+  return table[min(lane_id(), max(num_segments, 1) - 1)];
+}
+__device__ __forceinline__ int64_t segment_entry(int64_t preloaded, const int64_t* __restrict__ table, int seg) {
+  if (seg >= kWave) return table[seg];
+  const int src = __builtin_amdgcn_readfirstlane(seg);
+  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(preloaded)), src);
+  const uint32_t hi = __builtin_amdgcn_readlane(static_cast<int>(static_cast<uint64_t>(preloaded) >> 32), src);
+  return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 }  // namespace lorax

@@ -147,6 +147,16 @@ class LoraLinear(nn.Module):
         # them all) shrink together, as many per launch as fit a summed rank of 128 - x is read once per
         # launch; the reference issues one shrink per projection (utils/layers.py:121-133).
         for (r, _), group in prefill_jobs.items():
+            if _native.sgmv_lora_fits(r, input.size(1), input.size(0)):
+                # a short batch is bound by launches: shrink and expand of up to four projections in one
+                step = _native.MAX_FUSED_BGMV_PROBLEMS
+                for i in range(0, len(group), step):
+                    first = group[i][0]
+                    _native.sgmv_lora_multi(
+                        [(result, rs.lora_a_t_ptr, rs.lora_b_t_ptr, start, width) for rs, start, width in group[i : i + step]],
+                        input, first.segment_starts, first.segment_ends, r, self.layer_id,
+                    )
+                continue
             step = max(1, min(MAX_SGMV_SHRINK_PROBLEMS, MAX_RANK_CUSTOM // r))
             for i in range(0, len(group), step):
                 chunk = group[i : i + step]

@@ -95,6 +95,21 @@ def test_sgmv_shrink_multi_validation():
     assert f(two, 2, P, P, P, 0, 1000, 4096, 64, 0, 1.0, 0, P, 4 * big, 1, None) == OK  # a larger scratch is accepted
 
 
+def test_sgmv_lora_multi_validation():
+    f = _native.lib().lorax_sgmv_lora_multi
+    one = (_native.SgmvLoraProblem * 1)(_native.SgmvLoraProblem(P, P, P, 0, 4096, 4096))
+    assert f(one, 0, P, P, P, 2, 64, 4096, 16, 0, 1.0, 1, None) == EINVAL and "num_problems" in _err()
+    assert f(one, 1, P, P, P, 0, 64, 4096, 16, 0, 1.0, 1, None) == OK  # no segments
+    assert f(one, 1, P, P, None, 2, 64, 4096, 16, 0, 1.0, 1, None) == EINVAL and "null" in _err()
+    assert f(one, 1, P, P, P, 2, 64, 4096, 32, 0, 1.0, 1, None) == ENOKERNEL  # rank
+    assert f(one, 1, P, P, P, 2, 513, 4096, 16, 0, 1.0, 1, None) == ENOKERNEL  # too many rows
+    assert f(one, 1, P, P, P, 2, 64, 4096, 16, -1, 1.0, 1, None) == EINVAL
+    narrow = (_native.SgmvLoraProblem * 1)(_native.SgmvLoraProblem(P, P, P, 8, 4096, 4096))
+    assert f(narrow, 1, P, P, P, 2, 64, 4096, 16, 0, 1.0, 1, None) == EINVAL and "y_offset" in _err()
+    no_b = (_native.SgmvLoraProblem * 1)(_native.SgmvLoraProblem(P, P, None, 0, 4096, 4096))
+    assert f(no_b, 1, P, P, P, 2, 64, 4096, 16, 0, 1.0, 1, None) == EINVAL
+
+
 def test_sgmv_expand_validation():
     f = _native.lib().lorax_sgmv_expand
     for layout in (_native.B_RH, _native.B_HR):

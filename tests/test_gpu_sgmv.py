@@ -430,3 +430,55 @@ def test_sgmv_shrink_multi(dtype, count, r, h_in, lens):
         assert_close(vs[p], v_ref, f"projection {p}")
         assert_close(vs[p], singles[p].cpu(), f"projection {p} against its own launch")
         assert torch.count_nonzero(vs[p].cpu()[~covered]) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("r,h_in,widths,lens", [
+    (16, 4096, [4096], [16, 16, 16, 16]),          # the 64-token q_proj prefill
+    (8, 4096, [4096, 1024, 1024], [5, 0, 1, 33]),  # q/k/v slices of one fused output, an empty segment
+    (16, 1024, [520, 2048], [1, 1, 1, 1, 1, 1, 1]),  # ragged width, single-row segments
+    (8, 2048, [256], [130, 3, 200]),                # a few hundred rows
+])
+def test_sgmv_lora_single_launch(dtype, r, h_in, widths, lens):
+    """lorax_sgmv_lora_multi: shrink and expand of a short prefill batch in one launch - the values of the
+    overwrite-mode shrink followed by the transposed-B expand (the two paths add in different orders, so not
+    always the same bits) and the oracle's values."""
+    print(f"case dtype={dtype} r={r} h_in={h_in} widths={widths} lens={lens}", flush=True)
+    gen = torch.Generator().manual_seed(r + h_in + len(lens))
+    starts, ends, pos = [], [], 1
+    for n in lens:
+        starts.append(pos)
+        ends.append(pos + n)
+        pos += n + 1  # one uncovered row after every segment
+    T, layer = pos, 1
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    y0 = randn((T, sum(widths)), 0.5, gen, dtype, DEV)
+    s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
+    a_stacks = [[randn((2, r, h_in), 0.05, gen, dtype, DEV) if n > 0 else None for n in lens] for _ in widths]
+    b_stacks = [[randn((2, w, r), 0.05, gen, dtype, DEV) if n > 0 else None for n in lens] for w in widths]
+    a_tabs = [ptr_table(s, DEV) for s in a_stacks]
+    b_tabs = [ptr_table(s, DEV) for s in b_stacks]
+    offs = [sum(widths[:i]) for i in range(len(widths))]
+    y = y0.clone()
+    _native.sgmv_lora_multi([(y, a, b, off, w) for a, b, off, w in zip(a_tabs, b_tabs, offs, widths)], x, s_start, s_end,
+                            r, layer)
+    y2 = y0.clone()
+    scratch = sgmv.get_shrink_scratch(torch.device(DEV))
+    tmp = sgmv.get_tmp_tensor_for_size(len(lens), torch.device(DEV))
+    for a, b, off, w in zip(a_tabs, b_tabs, offs, widths):
+        v = sgmv.lora_a_sgmv_resident(x, scratch, a, s_start, s_end, layer, r, zero_fill=False)
+        sgmv.lora_b_sgmv_cutlass_slice(y2, v, tmp, b, s_start, s_end, layer, off, w, transposed=True)
+    torch.cuda.synchronize()
+    assert_close(y, y2.cpu(), "single launch against shrink + expand")
+    y_ref = y0.cpu().clone()
+    for p, (off, w) in enumerate(zip(offs, widths)):
+        for i, (s, e) in enumerate(zip(starts, ends)):
+            if e > s:
+                v_ref = (x.cpu()[s:e] @ a_stacks[p][i][layer].cpu().t())
+                y_ref[s:e, off:off + w] += (v_ref @ b_stacks[p][i][layer].cpu().t())
+    assert_close(y, y_ref, "y")
+    covered = torch.zeros(T, dtype=torch.bool)
+    for s, e in zip(starts, ends):
+        covered[s:e] = True
+    assert torch.equal(y.cpu()[~covered], y0.cpu()[~covered])
