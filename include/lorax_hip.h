@@ -72,7 +72,8 @@ extern "C" {
  *
  * h_in < h_out selects "expand" (h_in is the LoRA rank), otherwise "shrink"
  * (h_out is the rank), as bgmv_impl.cuh:204.  The rank must be a multiple of 8 in
- * [8, 128]; the wide dimension a multiple of 8 below 65536 (punica_ops.cc:310).
+ * [8, 128]; the wide dimension a multiple of 8, below 65536 for a shrink (punica_ops.cc:310) and
+ * below 2^20 for an expand (so that the LM head of a large-vocabulary model is served too).
  * The reference binds y_offset = 0 and y_stride = h_out (punica_ops.cc:318); other
  * values let a caller write one projection's slice of a fused q/k/v or gate/up
  * output in place.

@@ -467,10 +467,12 @@ def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: floa
 SGMV_LORA_MAX_TOKENS = 512
 
 
-def sgmv_lora_fits(rank: int, h_in: int, num_tokens: int) -> bool:
+def sgmv_lora_fits(rank: int, h_in: int, num_tokens: int, h_out: int = 0) -> bool:
     """True where the single-launch prefill update (lorax_sgmv_lora_multi) applies and pays: rank 8 or 16 with a
-    small A slab, and a batch short enough to be bound by launches."""
-    return rank in FUSED_BGMV_RANKS and rank * h_in * 2 <= 128 * 1024 and num_tokens <= SGMV_LORA_MAX_TOKENS
+    small A slab, a batch short enough to be bound by launches, and an output that is not so wide (an LM head)
+    that recomputing the shrink in every column slice would dominate."""
+    return (rank in FUSED_BGMV_RANKS and rank * h_in * 2 <= 128 * 1024 and num_tokens <= SGMV_LORA_MAX_TOKENS
+            and h_out <= 16384)
 
 
 def sgmv_lora_multi(problems, x, s_start, s_end, rank, layer_idx, scale: float = 1.0) -> None:

@@ -288,8 +288,10 @@ class BatchLoraWeights(BatchAdapterWeights):
         return adapter_index in self.adapter_index_configs
 
     def can_vectorize(self, pg) -> bool:
-        within = all(rd.rank // pg.size() <= MAX_RANK_CUSTOM for rd in self.rank_data.values())
-        return within and self.layer_name != LM_HEAD
+        """True when the kernels serve every rank group.  The reference also returns False for the LM head
+        (adapters/lora.py:243-247: its BGMV kernels stop at 65 535 output columns) and runs its dense loop
+        there; the kernels here take vocabulary-wide outputs, so the LM head is served like any projection."""
+        return all(rd.rank // pg.size() <= MAX_RANK_CUSTOM for rd in self.rank_data.values())
 
     @classmethod
     def key(cls) -> str:
@@ -504,16 +506,20 @@ class AdapterBatchData:
         prefill: bool = False,
         prefill_head_indices: Optional[torch.Tensor] = None,
     ) -> "AdapterBatchData":
-        data = _native_batch_tables(meta, weights, prefill) if prefill_head_indices is None else None
-        if data is None:
-            data = {}
-            for layer_name, layer_weights in weights.items():
-                if layer_weights.is_empty():
-                    continue
-                head = prefill_head_indices if layer_name == LM_HEAD else None
-                batched = layer_weights.get_data(meta, layer_name, prefill, head)
-                if batched:
-                    data[layer_name] = batched
+        # The native builder makes the tables of all layer types in one call; the LM head of a prefill batch,
+        # whose input rows are requests rather than tokens, keeps the per-layer-type Python path.
+        head_rows = prefill_head_indices is not None
+        native_names = {n: w for n, w in weights.items() if not (head_rows and n == LM_HEAD)}
+        data = _native_batch_tables(meta, native_names, prefill)
+        remaining = weights if data is None else {n: w for n, w in weights.items() if n not in native_names}
+        data = {} if data is None else data
+        for layer_name, layer_weights in remaining.items():
+            if layer_weights.is_empty():
+                continue
+            head = prefill_head_indices if layer_name == LM_HEAD else None
+            batched = layer_weights.get_data(meta, layer_name, prefill, head)
+            if batched:
+                data[layer_name] = batched
         return AdapterBatchData(
             meta=meta,
             data=data,

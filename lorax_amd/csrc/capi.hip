@@ -136,9 +136,11 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
     const bool expand = q_in < h_out;
     const int narrow = expand ? q_in : h_out;
     const int wide = expand ? h_out : q_in;
-    // punica_ops.cc:310 (dims < 65536) and bgmv_config.h:12-86 (narrow side 8..128).
-    if (q_in <= 0 || h_out <= 0 || q_in >= 65536 || h_out >= 65536 || narrow % 8 != 0 ||
-        narrow > kMaxRank || wide % 8 != 0)
+    // bgmv_config.h:12-86 (narrow side 8..128).  The reference also wants both dims below 65536
+    // (punica_ops.cc:310), which shuts out the LM head of models with large vocabularies and sends it to the
+    // dense loop; here the wide side of an expand may be up to 2^20.
+    const int wide_limit = expand ? (1 << 20) : 65536;
+    if (q_in <= 0 || h_out <= 0 || wide >= wide_limit || narrow % 8 != 0 || narrow > kMaxRank || wide % 8 != 0)
       return fail(LORAX_ENOKERNEL, "No suitable kernel. h_in=%d h_out=%d dtype=%d", q_in, h_out, dtype);
     if (expand != a.expand)
       return fail(LORAX_EINVAL, "problems of one launch must share the direction (problem %d: h_in=%d h_out=%d)", i,

@@ -15,6 +15,8 @@ Deliberate differences from the reference:
     group, so both orders round identically;
   * in prefill the shrink overwrites the rows of the segments in v, so v is not zero-filled first
     (utils/punica.py:176-178 allocates zeros); the expand reads no other rows;
+  * the LM head takes the same kernels (MultiAdapterHead): the reference excludes it from its kernel path
+    (adapters/lora.py:243-247) and runs the dense loop, because its BGMV kernels stop at 65 535 columns;
   * in decode, the projections of one layer that share an input (q/k/v, gate/up) go to the
     GPU as ONE shrink launch and ONE expand launch per rank (``lorax_bgmv_multi``), and the
     shrink overwrites v, so there is no zero-fill (:146).  A decode-size BGMV is shorter
@@ -70,7 +72,7 @@ class LoraLinear(nn.Module):
         if not data.can_vectorize(self.process_group):
             raise RuntimeError(
                 f"layer type {layer_type!r}: ranks {sorted(data.rank_data)} are outside what the LoRA kernels "
-                "cover (rank / world_size <= 128, not lm_head)"
+                "cover (rank / world_size <= 128)"
             )
         return data
 
@@ -147,7 +149,7 @@ class LoraLinear(nn.Module):
         # them all) shrink together, as many per launch as fit a summed rank of 128 - x is read once per
         # launch; the reference issues one shrink per projection (utils/layers.py:121-133).
         for (r, _), group in prefill_jobs.items():
-            if _native.sgmv_lora_fits(r, input.size(1), input.size(0)):
+            if _native.sgmv_lora_fits(r, input.size(1), input.size(0), max(width for _, _, width in group)):
                 # a short batch is bound by launches: shrink and expand of up to four projections in one
                 step = _native.MAX_FUSED_BGMV_PROBLEMS
                 for i in range(0, len(group), step):
@@ -287,3 +289,13 @@ class TensorParallelAdapterRowLinear(LoraLinear):
         start = self.process_group.rank() * stride
         self.forward_layer_type(result, input, adapter_data, self.layer_name, start, start + stride)
         return result
+
+
+class MultiAdapterHead(TensorParallelAdapterRowLinear):
+    """The LM head with LoRA (utils/layers.py:303-326).  In a prefill batch its input holds one row per request
+    (the last token's hidden state); BatchLoraWeights.load has recounted the segment bounds in those rows from
+    prefill_head_indices, so the same kernels apply.  Returns (logits, speculative_logits); the Medusa heads
+    that would fill the second slot are not part of this package, so it is always None."""
+
+    def forward(self, input: torch.Tensor, adapter_data: AdapterBatchData):
+        return super().forward(input, adapter_data), None

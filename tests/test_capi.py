@@ -52,7 +52,7 @@ def test_bgmv_validation():
     assert f(None, P, P, P, 4, 4096, 8, 0, 8, 0, 1.0, 1, None) == EINVAL and "null" in _err()
     assert f(P, P + 2, P, P, 4, 4096, 8, 0, 8, 0, 1.0, 1, None) == EINVAL and "aligned" in _err()
     assert f(P, P, P, P, 4, 4096, 8, 0, 8, 0, 1.0, 2, None) == ENOKERNEL and "No suitable kernel" in _err()
-    for h_in, h_out in [(4096, 12), (4096, 136), (4100, 8), (65536, 8), (8, 65536), (256, 256)]:
+    for h_in, h_out in [(4096, 12), (4096, 136), (4100, 8), (65536, 8), (8, 1 << 20), (256, 256)]:
         assert f(P, P, P, P, 4, h_in, h_out, 0, h_out, 0, 1.0, 1, None) == ENOKERNEL, (h_in, h_out)
         assert f"h_in={h_in} h_out={h_out}" in _err()
     assert f(P, P, P, P, 4, 8, 4096, 8192, 8192, 0, 1.0, 1, None) == EINVAL  # window outside the row

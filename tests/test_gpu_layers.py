@@ -149,3 +149,48 @@ def test_config5_mlp_projections_reduced():
                           num_adapters=6, groups=groups)
     assert_has_empty_segments(w, w.batch_data())
     _check_workload(w, 0, 0.25)
+
+
+@pytest.mark.parametrize("prefill", [True, False])
+def test_lm_head_with_a_large_vocabulary(prefill):
+    """The LM head through MultiAdapterHead: 70 000 output columns (more than the reference's BGMV kernels take),
+    adapters of rank 8 and 16 and requests without adapter.  In prefill the head sees one row per request, picked
+    by prefill_head_indices, and the segment bounds are recounted in those rows."""
+    from lorax_amd.adapters import LM_HEAD, AdapterBatchData, LayerAdapterWeights, LoraConfig, LoraWeights
+    from lorax_amd.layers import MultiAdapterHead
+    from lorax_amd.synthetic import make_meta
+
+    dtype, hidden, vocab = torch.bfloat16, 1024, 70000
+    gen = torch.Generator().manual_seed(5)
+    request_adapters = [0, 0, 1, 7, 1, 2, 2, 2, 7, 0]      # 7 has no weights
+    lens = [5, 1, 9, 3, 2, 6, 1, 4, 2, 8] if prefill else [1] * len(request_adapters)
+    tokens = [a for a, n in zip(request_adapters, lens) for _ in range(n)]
+    meta = make_meta(tokens, torch.device(DEV))
+    head_idx = None
+    if prefill:
+        ends = torch.tensor(lens).cumsum(0)
+        head_idx = (ends - 1).to(torch.int64).to(DEV)  # last token of every request
+    layer = LayerAdapterWeights()
+    ranks = {0: 8, 1: 16, 2: 16}
+    for a, r in ranks.items():
+        wa = (torch.randn((1, hidden, r), generator=gen) * 0.05).to(dtype).to(DEV)
+        wb = (torch.randn((1, r, vocab), generator=gen) * 0.05).to(dtype).to(DEV)
+        layer.add_adapter(a, LoraWeights(list(wa.unbind(0)), list(wb.unbind(0)), LoraConfig(r=r)))
+    batch = AdapterBatchData.from_meta(meta, {LM_HEAD: layer}, prefill=prefill, prefill_head_indices=head_idx)
+    rows = len(request_adapters)
+    x = (torch.randn((rows, hidden), generator=gen)).to(dtype)
+    y0 = (torch.randn((rows, vocab), generator=gen) * 0.25).to(dtype)
+    head = MultiAdapterHead.load(ZeroBase(y0.to(DEV)), 0, LM_HEAD)
+    logits, speculative = head(x.to(DEV), batch)
+    torch.cuda.synchronize()
+    assert speculative is None
+    ref = y0.clone()
+    idx = torch.tensor(request_adapters)
+    lora_a = {a: lw.weights_a.cpu() for a, lw in layer.adapter_weights.items()}
+    lora_b = {a: lw.weights_b.cpu() for a, lw in layer.adapter_weights.items()}
+    O.fallback_layer_type(ref, x, idx, set(request_adapters), lora_a, lora_b, 0, 0, vocab)
+    delta = (ref.float() - y0.float()).to(dtype)
+    assert_close(logits, ref, "lm_head logits", rounded=[delta])
+    untouched = torch.tensor([a not in ranks for a in request_adapters])
+    assert torch.equal(logits.cpu()[untouched], y0[untouched])
+    assert torch.count_nonzero(logits.cpu()[~untouched] != y0[~untouched]) > 0
