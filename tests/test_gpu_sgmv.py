@@ -194,12 +194,14 @@ def test_sgmv_expand_transposed_b(dtype, r, h_out, lens, window):
             delta = v.cpu()[s:e] @ wb[i][layer].cpu()
             y_ref[s:e, off:off + width] = y_ref[s:e, off:off + width] + delta
     assert_close(y_t, y_ref, "transposed-B expand", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
-    # Segments of more than 4 rows run the same MFMA arithmetic in the same order for both layouts (the
-    # reference-layout kernel sums shorter ones on the vector ALU).
+    # Row tiles of more than 4 rows run the same MFMA arithmetic in the same order for both layouts (the
+    # reference-layout kernel sums shorter ones on the vector ALU); a segment is cut into tiles of 256 rows.
     long_rows = torch.zeros(T, dtype=torch.bool)
     for s, e in zip(starts, ends):
-        if e - s > 4:
-            long_rows[s:e] = True
+        full = s + (e - s) // 256 * 256
+        long_rows[s:full] = True
+        if e - full > 4:
+            long_rows[full:e] = True
     assert torch.equal(y_t.cpu()[long_rows], y_n.cpu()[long_rows])
     assert_close(y_n, y_ref, "reference-layout expand", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
     outside = torch.ones_like(y0, dtype=torch.bool).cpu()
