@@ -58,7 +58,8 @@ template <typename D, int NB, int MBLK, bool KSPLIT>
 __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     const ShrinkGroup grp, const typename D::E* __restrict__ X, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int64_t layer_idx,
-    int stages, float scale, int accumulate_into_v, int rows_per_tile) {
+    int stages, float scale, int accumulate_into_v, int rows_per_tile, int kparts, int tile_slots,
+    float* __restrict__ partials) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   // The A tile stacks the A matrices of grp.count projections of rank r: row p * r + i is row i of
@@ -94,9 +95,17 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
   const int wm = KSPLIT ? 0 : wave % WM;
   const int wn = KSPLIT ? 0 : wave / WM;
   const VirtualBlock vb = xcd_virtual_block();
-  const int nst = h_in / kLdsKc;
+  // K split across workgroups (kparts > 1, launches with few row tiles): workgroup p * tile_slots + t multiplies
+  // part p of the hidden dimension for tile t and leaves its fp32 sums in partials[p][row][R]; a second kernel
+  // adds the parts in a fixed order.  Tiles are numbered fastest: neighbours (one XCD) read the same part of A.
+  const int kpart = kparts > 1 ? vb.x / tile_slots : 0;
+  const int first_tile = kparts > 1 ? vb.x - kpart * tile_slots : vb.x;
+  const int st_begin = static_cast<int>(static_cast<int64_t>(kpart) * (h_in / kLdsKc) / kparts);
+  const int nst = static_cast<int>(static_cast<int64_t>(kpart + 1) * (h_in / kLdsKc) / kparts) - st_begin;
+  const int k_begin = st_begin * kLdsKc;
 
-  for (int tile = vb.x;; tile += gridDim.x) {
+  for (int tile = first_tile;; tile += gridDim.x) {
+    if (kparts > 1 && tile != first_tile) break;  // one tile per workgroup when K is split
     RowTile rt;
     // tiles may be lower than the ROWS the buffers hold: rows past a tile's end re-read its last row
     if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
@@ -114,7 +123,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
       const int id = j * kLdsThreads + tid;
       const int row = id >> 4;
       const int grow = min(rt.row0 + row, rt.row_end - 1);  // rows past the tile re-read its last row
-      xsrc[j] = X + static_cast<int64_t>(grow) * h_in + (((id & 15) ^ (row & 15)) << 3);
+      xsrc[j] = X + static_cast<int64_t>(grow) * h_in + k_begin + (((id & 15) ^ (row & 15)) << 3);
     }
 #pragma unroll
     for (int j = 0; j < kALoads; ++j) {
@@ -123,7 +132,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
       int proj = row / r, arow = row - proj * r;
       if (proj >= grp.count) proj = grp.count - 1, arow = r - 1;
       const E* Ap = proj == 0 ? A[0] : (proj == 1 ? A[1] : (proj == 2 ? A[2] : A[3]));
-      asrc[j] = Ap + static_cast<int64_t>(arow) * h_in + (((id & 15) ^ (row & 15)) << 3);
+      asrc[j] = Ap + static_cast<int64_t>(arow) * h_in + k_begin + (((id & 15) ^ (row & 15)) << 3);
     }
     auto issue = [&](int st, int slot) {
       char* buf = lds + slot * kStageBytes;
@@ -183,7 +192,10 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     // Four adjacent columns of one row (r is a multiple of 8: they belong to one projection).
     auto store4 = [&](int row, int col, f32x4 sum) {
       const int proj = col / r;
-      if (row < rt.row_end && proj < grp.count) {
+      if (kparts > 1) {
+        if (row < rt.row_end && proj < grp.count)
+          *reinterpret_cast<f32x4*>(partials + (static_cast<int64_t>(kpart) * num_tokens + row) * R + col) = sum;
+      } else if (row < rt.row_end && proj < grp.count) {
         E* Vp = static_cast<E*>(proj == 0 ? grp.v[0] : (proj == 1 ? grp.v[1] : (proj == 2 ? grp.v[2] : grp.v[3])));
         update4<D>(accumulate_into_v != 0, Vp + static_cast<int64_t>(row) * r + (col - proj * r), sum * scale);
       }
@@ -227,6 +239,36 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
   }
 }
 
+// Second pass of a launch that split K across workgroups: adds the parts of every row of every tile in a fixed
+// order and finishes the row exactly as the one-pass kernel does (scale, round, add or overwrite).
+template <typename D>
+__global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_parts_kernel(
+    const ShrinkGroup grp, const float* __restrict__ partials, const int32_t* __restrict__ s_start,
+    const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int R, int kparts, float scale,
+    int accumulate_into_v, int rows_per_tile) {
+  using E = typename D::E;
+  const int r = grp.rank;
+  const int n4 = grp.count * r / 4;  // groups of 4 adjacent columns per row (r is a multiple of 8)
+  for (int tile = blockIdx.x;; tile += gridDim.x) {
+    RowTile rt;
+    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
+    const int n = (rt.row_end - rt.row0) * n4;
+    for (int i = threadIdx.x; i < n; i += kLdsThreads) {
+      const int row = rt.row0 + i / n4;
+      const int col = (i % n4) * 4;
+      f32x4 sum = *reinterpret_cast<const f32x4*>(partials + static_cast<int64_t>(row) * R + col);
+      for (int p = 1; p < kparts; ++p) {
+        const f32x4 part =
+            *reinterpret_cast<const f32x4*>(partials + (static_cast<int64_t>(p) * num_tokens + row) * R + col);
+        sum[0] += part[0]; sum[1] += part[1]; sum[2] += part[2]; sum[3] += part[3];
+      }
+      const int proj = col / r;
+      E* Vp = static_cast<E*>(proj == 0 ? grp.v[0] : (proj == 1 ? grp.v[1] : (proj == 2 ? grp.v[2] : grp.v[3])));
+      update4<D>(accumulate_into_v != 0, Vp + static_cast<int64_t>(row) * r + (col - proj * r), sum * scale);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------
@@ -247,10 +289,28 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
     rows_per_tile = (tuning().shrink_rows + 15) / 16 * 16;
   }
   const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
+  // K parts: a workgroup streams its tile's x and A at about 50 GB/s whatever the launch, so a launch of a
+  // hundred tiles (a prefill batch of one or two thousand rows) leaves most of the chip idle.  Its hidden
+  // dimension is cut into parts of at least 8 stages, about one workgroup per CU (two measured no faster), and a
+  // second small launch adds the parts.  Needs the scratch (fp32 sums, kparts x rows x R); decided from
+  // host-known sizes only.
+  constexpr int R = NB * 16;
+  int kparts = 1;
+  const int nst_all = a.d_in / kLdsKc;
+  if (a.partials != nullptr && (tiles <= 128 || tuning().shrink_ksplit > 0)) {
+    kparts = static_cast<int>(256 / tiles);
+    if (kparts > 8) kparts = 8;
+    if (kparts > nst_all / 8) kparts = nst_all / 8;
+    if (tuning().shrink_ksplit > 0) kparts = tuning().shrink_ksplit < nst_all ? tuning().shrink_ksplit : nst_all;
+    const size_t room = a.partial_bytes < kPartialBytes ? a.partial_bytes : kPartialBytes;
+    while (kparts > 1 && static_cast<size_t>(kparts) * a.num_tokens * R * sizeof(float) > room) --kparts;
+    if (kparts < 1) kparts = 1;
+  }
+  const int64_t wgs = tiles * kparts;
   // Stage buffers: all of a CU's LDS when there is at most one workgroup per CU; a third of it when the
-  // tiles make one to three rounds over the CUs (more resident workgroups even out the last round);
+  // workgroups make one to three rounds over the CUs (more resident workgroups even out the last round);
   // half of it for long launches.  2 to 8 stages.
-  int budget = tiles <= 256 ? 150 * 1024 : (tiles <= 768 ? 50 * 1024 : 76 * 1024);
+  int budget = wgs <= 256 ? 150 * 1024 : (wgs <= 768 ? 50 * 1024 : 76 * 1024);
   if (tuning().shrink_lds_kb > 0) budget = tuning().shrink_lds_kb * 1024;
   int stages = budget / kStageBytes;
   stages = stages < 2 ? 2 : (stages > kLdsMaxStages ? kLdsMaxStages : stages);
@@ -270,7 +330,7 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     if (device >= 0 && device < 64) configured[device] = true;
   }
-  dim3 grid(static_cast<unsigned>(tiles < (1 << 20) ? tiles : (1 << 20)));
+  dim3 grid(static_cast<unsigned>(kparts > 1 ? wgs : (tiles < (1 << 20) ? tiles : (1 << 20))));
   ShrinkGroup grp = a.group;
   if (grp.count <= 1) {
     grp = ShrinkGroup{};
@@ -281,7 +341,12 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, grp, static_cast<const typename D::E*>(a.x),
                      a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages,
-                     a.scale, a.accumulate, rows_per_tile);
+                     a.scale, a.accumulate, rows_per_tile, kparts, static_cast<int>(tiles), a.partials);
+  e = hipGetLastError();
+  if (e != hipSuccess || kparts == 1) return e;
+  hipLaunchKernelGGL(sgmv_shrink_parts_kernel<D>, dim3(static_cast<unsigned>(tiles)), dim3(kLdsThreads), 0, stream, grp,
+                     a.partials, a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), R, kparts, a.scale,
+                     a.accumulate, rows_per_tile);
   return hipGetLastError();
 }
 

@@ -135,6 +135,9 @@ def test_sgmv_shrink_expand_vs_oracle(dtype, r, h_in, h_out, lens):
     (48, 256, [600, 700, 800, 900, 1000]),    # 32-row tiles, odd number of rank blocks
     (128, 256, [40] * 100 + [1] * 60),        # 32-row tiles, rank 128, many short segments
     (16, 128, [1] * 600),                     # 16-row tiles, one row each
+    (64, 4096, [200, 300, 7, 400, 100]),      # a thousand rows: hidden dimension in 3 parts, second pass adds them
+    (128, 2048, [600, 1, 50]),                # the same at rank 128, 2 parts
+    (40, 3072, [513]),                        # the same with an odd number of rank blocks, one segment
     (64, 192, [3000, 2000, 3000]),            # h_in not a multiple of 128: register-operand kernel
     (16, 4160, [330, 290]),                   # the same with K split across workgroups
     (24, 1000, [100, 28, 1]),                 # a few rows: streaming kernel, any rank and h_in multiple of 8
@@ -386,6 +389,7 @@ def test_sgmv_errors_raise_runtime_error():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("count,r,h_in,lens", [
     (2, 64, 1024, [700, 1, 0, 33, 1, 300]),   # gate/up at rank 64: one launch of summed rank 128
+    (2, 64, 4096, [500, 1, 0, 33, 1, 300]),   # the same with the hidden dimension cut into parts (two passes)
     (3, 16, 512, [520, 17, 64]),              # q/k/v at rank 16
     (3, 40, 256, [1, 600, 5]),                # summed rank 120, not a multiple of 16 per projection
     (4, 8, 384, [256, 257, 3]),               # four projections of rank 8
