@@ -161,9 +161,9 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
  *
  * `tmp`/`tmp_bytes` is the caller's scratch, with the reference's sizes (8 MiB for LORAX_A_RH, punica_ops.cc:
  * 389-390; lorax_sgmv_tmp_size(num_segments) for LORAX_A_HR, punica_ops.cc:359).  For LORAX_A_RH the launch
- * may write it (fp32 partial sums and arrival counters when K is split across workgroups: h_in not a multiple
- * of 128 and a few hundred to a few thousand rows); nothing is expected in it on entry and nothing of value is
- * left in it.  As in the reference, two shrinks that are in flight at the same time (different streams) must
+ * may write it (fp32 partial sums, and arrival counters, when the hidden dimension is split across workgroups:
+ * batches of roughly 500 to 2000 rows, and h_in that is not a multiple of 128); nothing is expected in it on
+ * entry and nothing of value is left in it.  As in the reference, two shrinks that are in flight at the same time (different streams) must
  * not share one tmp buffer.
  */
 int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
@@ -179,10 +179,11 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
  * inside the library's own device image, one copy per GPU, held until the process ends; its address on a
  * device is looked up on the first call there (or by lorax_init).
  *
- * Limit: a call served by the split-K kernel (LORAX_A_RH, h_in not a multiple of 128, more than 512 rows) needs
- * 2 * num_tokens * r * 4 bytes <= LORAX_SHRINK_TMP_BYTES - 65536, i.e. room for two fp32 partial tiles of the
- * batch; beyond that the call fails with LORAX_ESPACE and launches nothing.  Other shapes use no scratch and
- * have no limit.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * Limit: a call served by the register-operand kernel (LORAX_A_RH, h_in not a multiple of 128, more than 512
+ * rows) needs 2 * num_tokens * r * 4 bytes <= LORAX_SHRINK_TMP_BYTES - 65536, i.e. room for two fp32 partial
+ * tiles of the batch; beyond that the call fails with LORAX_ESPACE and launches nothing.  Other shapes have no
+ * limit: they use no scratch, or (h_in a multiple of 128, about 500 to 2000 rows) split the hidden dimension
+ * only as far as the array has room for.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
  * streams or threads) race; calls on one stream, or ordered by events, do not.  Nothing needs to be cleared
  * between calls (the arrival counters are cleared by every launch that uses them).
  */
@@ -199,8 +200,9 @@ int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, cons
  * multiple of 128 and the batch has more than 512 rows, the projections run as ONE launch that reads x once
  * (their A matrices are stacked into one rank-(num_problems * r) tile).  Otherwise the call issues one
  * launch per projection.  `tmp`/`tmp_bytes`: at least LORAX_SHRINK_TMP_BYTES of scratch, as for lorax_sgmv_shrink
- * with LORAX_A_RH; a larger buffer is accepted (a launch that splits K across workgroups keeps its fp32 partial
- * sums there and can split further the more room it has).  num_problems = 1 is allowed.
+ * with LORAX_A_RH; a larger buffer is accepted and changes nothing (a launch that splits the hidden dimension
+ * across workgroups keeps its fp32 partial sums in the first 8 MiB, so that the result does not depend on the
+ * buffer's size).  num_problems = 1 is allowed.
  * accumulate = 1 adds to v as lorax_sgmv_shrink does; accumulate = 0 stores dtype(scale * x @ A^T) into the rows
  * of the segments instead, so the caller need not zero v first (rows outside every segment keep their contents;
  * lorax_sgmv_expand reads no others).  The reference zero-fills v before every shrink (punica.py:176-178).
