@@ -68,7 +68,9 @@ __global__ __launch_bounds__(kExpandThreads) void sgmv_expand_kernel(
 
   for (int tile = blockIdx.y;; tile += gridDim.y) {
     RowTile rt;
-    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
+    // small remainders are merged into the segment's other tiles: a tile's prologue (search, staging the panels)
+    // costs as much as a hundred rows
+    if (!find_row_tile<true>(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const E* B = reinterpret_cast<const E*>(segment_entry(pre_w, W, rt.seg)) + layer_idx * r * static_cast<int64_t>(h_out);
     const int nrows = rt.row_end - rt.row0;
     if (nrows <= kExpandShortRows) {

@@ -83,7 +83,9 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
   const int64_t pre_w = preload_segment_entry(W, num_segments);
   for (int tile = vid % tile_slots;; tile += tile_slots) {
     RowTile rt;
-    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
+    // small remainders are merged into the segment's other tiles: a tile's prologue (the search and the panel
+    // operands) costs as much as a hundred rows
+    if (!find_row_tile<true>(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const E* BT = reinterpret_cast<const E*>(segment_entry(pre_w, W, rt.seg)) + layer_idx * h_out * static_cast<int64_t>(r);
     const int nmb = (rt.row_end - rt.row0 + 15) / 16;
 
@@ -175,9 +177,10 @@ static hipError_t launch_expand_t_ks(const SgmvArgs& a, hipStream_t stream) {
   // 256-row tiles: the prologue is one memory round trip, so taller tiles buy nothing and even out worse
   int rows_per_tile = 256;
   if (tuning().expand_rows > 0) rows_per_tile = (tuning().expand_rows + 15) / 16 * 16;
-  // the kernel addresses a tile with 32-bit element offsets
-  if (a.y_stride * rows_per_tile >= (1ll << 32) || static_cast<int64_t>(a.d_in) * rows_per_tile >= (1ll << 32))
-    return hipErrorInvalidValue;
+  // The kernel addresses a tile with 32-bit element offsets, and a tile is up to 9/8 * rows_per_tile + 15 rows
+  // high (merged remainders): rows of more than 2^23 elements get lower tiles.
+  while (rows_per_tile > 16 && a.y_stride * (rows_per_tile + rows_per_tile / 8 + 16) >= (1ll << 32)) rows_per_tile /= 2;
+  if (a.y_stride * (rows_per_tile + rows_per_tile / 8 + 16) >= (1ll << 32)) return hipErrorInvalidValue;
   const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
   constexpr int kCols = 16 * NJ;
   const int num_panels = (a.d_out + kCols - 1) / kCols;

@@ -21,11 +21,22 @@ struct RowTile {
 // One chunk of 64 segments: lane `lane` holds the clamped bounds (s, e) of segment seg0 + lane.  If `tile`
 // (counted from the first tile of the chunk, `rel`) falls into the chunk, fills `out` and returns true;
 // otherwise adds the chunk's tiles to `base`.
+// MERGE: a remainder that would make the segment's full tiles at most an eighth taller is shared out among them
+// instead of becoming a tile of its own, and the segment's tiles get equal heights (in 16-row blocks).  For
+// kernels whose tile prologue is expensive (a batch of 269-row segments cost the expand 38 % more than one of
+// 256-row segments) and whose tile height is free; taller tiles than that unbalance the end of the launch.
+__device__ __forceinline__ int merged_tile_count(int len, int rows_per_tile) {
+  const int full = len / rows_per_tile;
+  const int rem = len - full * rows_per_tile;
+  return (full >= 1 && rem * 8 <= full * rows_per_tile) ? full : full + (rem > 0 ? 1 : 0);
+}
+
+template <bool MERGE = false>
 __device__ __forceinline__ bool tile_in_chunk(int s, int e, int seg0, int rows_per_tile, int tile, int& base,
                                               RowTile& out) {
   const int lane = lane_id();
   const int len = max(e - s, 0);
-  const int nt = (len + rows_per_tile - 1) / rows_per_tile;
+  const int nt = MERGE ? merged_tile_count(len, rows_per_tile) : (len + rows_per_tile - 1) / rows_per_tile;
   int inc = nt;
 #pragma unroll
   for (int d = 1; d < kWave; d <<= 1) {
@@ -42,8 +53,15 @@ __device__ __forceinline__ bool tile_in_chunk(int s, int e, int seg0, int rows_p
     const int s_f = __shfl(s, src, kWave);
     const int e_f = __shfl(e, src, kWave);
     out.seg = seg0 + src;
-    out.row0 = s_f + ti * rows_per_tile;
-    out.row_end = min(e_f, out.row0 + rows_per_tile);
+    if (MERGE) {
+      const int nt_f = __shfl(nt, src, kWave);
+      const int blocks = (e_f - s_f + 15) / 16;
+      out.row0 = s_f + 16 * static_cast<int>(static_cast<int64_t>(ti) * blocks / nt_f);
+      out.row_end = min(e_f, s_f + 16 * static_cast<int>(static_cast<int64_t>(ti + 1) * blocks / nt_f));
+    } else {
+      out.row0 = s_f + ti * rows_per_tile;
+      out.row_end = min(e_f, out.row0 + rows_per_tile);
+    }
     return true;
   }
   base += chunk_total;
@@ -56,6 +74,7 @@ __device__ __forceinline__ bool tile_in_chunk(int s, int e, int seg0, int rows_p
 // trip instead of one per 64 segments.
 constexpr int kTilePreload = 4;
 
+template <bool MERGE = false>
 __device__ __forceinline__ bool find_row_tile(const int32_t* __restrict__ s_start,
                                               const int32_t* __restrict__ s_end,
                                               int num_segments, int num_tokens,
@@ -77,7 +96,7 @@ __device__ __forceinline__ bool find_row_tile(const int32_t* __restrict__ s_star
     const bool live = c * kWave + lane < num_segments;
     const int s = live ? max(s_pre[c], 0) : 0;
     const int e = live ? min(e_pre[c], num_tokens) : 0;
-    if (tile_in_chunk(s, e, c * kWave, rows_per_tile, tile, base, out)) return true;
+    if (tile_in_chunk<MERGE>(s, e, c * kWave, rows_per_tile, tile, base, out)) return true;
   }
   for (int seg0 = kTilePreload * kWave; seg0 < num_segments; seg0 += kWave) {
     const int seg = seg0 + lane;
@@ -86,7 +105,7 @@ __device__ __forceinline__ bool find_row_tile(const int32_t* __restrict__ s_star
       s = max(s_start[seg], 0);
       e = min(s_end[seg], num_tokens);
     }
-    if (tile_in_chunk(s, e, seg0, rows_per_tile, tile, base, out)) return true;
+    if (tile_in_chunk<MERGE>(s, e, seg0, rows_per_tile, tile, base, out)) return true;
   }
   return false;
 }

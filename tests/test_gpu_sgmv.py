@@ -197,14 +197,13 @@ def test_sgmv_expand_transposed_b(dtype, r, h_out, lens, window):
             delta = v.cpu()[s:e] @ wb[i][layer].cpu()
             y_ref[s:e, off:off + width] = y_ref[s:e, off:off + width] + delta
     assert_close(y_t, y_ref, "transposed-B expand", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
-    # Row tiles of more than 4 rows run the same MFMA arithmetic in the same order for both layouts (the
-    # reference-layout kernel sums shorter ones on the vector ALU); a segment is cut into tiles of 256 rows.
+    # Segments of more than 4 rows run the same MFMA arithmetic in the same order for both layouts (the
+    # reference-layout kernel sums shorter ones on the vector ALU; a remainder of a few rows is merged into the
+    # segment's other tiles, so only segments of up to 4 rows make such tiles).
     long_rows = torch.zeros(T, dtype=torch.bool)
     for s, e in zip(starts, ends):
-        full = s + (e - s) // 256 * 256
-        long_rows[s:full] = True
-        if e - full > 4:
-            long_rows[full:e] = True
+        if e - s > 4:
+            long_rows[s:e] = True
     assert torch.equal(y_t.cpu()[long_rows], y_n.cpu()[long_rows])
     assert_close(y_n, y_ref, "reference-layout expand", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
     outside = torch.ones_like(y0, dtype=torch.bool).cpu()
