@@ -20,6 +20,8 @@
 // and one s_barrier (everybody's have; everybody is done with the buffer about to be refilled).
 // The barrier is a bare s_barrier: __syncthreads() would wait for ALL outstanding loads and
 // serialise the pipeline.
+#include <atomic>
+
 #include "kernels.h"
 #include "sgmv_tiles.h"
 
@@ -320,15 +322,15 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   if (lds_bytes < kRedBytes) lds_bytes = kRedBytes;
   auto kernel = sgmv_shrink_lds_kernel<D, NB, MBLK, KSPLIT>;
   // Raising the dynamic LDS limit is needed once per kernel and device.
-  static bool configured[64] = {};
+  static std::atomic<bool> configured[64] = {};  // callers may come from several host threads
   int device = 0;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return e;
-  if (device < 0 || device >= 64 || !configured[device]) {
+  if (device < 0 || device >= 64 || !configured[device].load(std::memory_order_acquire)) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             kLdsMaxBytes);
     if (e != hipSuccess) return e;
-    if (device >= 0 && device < 64) configured[device] = true;
+    if (device >= 0 && device < 64) configured[device].store(true, std::memory_order_release);
   }
   dim3 grid(static_cast<unsigned>(kparts > 1 ? wgs : (tiles < (1 << 20) ? tiles : (1 << 20))));
   ShrinkGroup grp = a.group;
