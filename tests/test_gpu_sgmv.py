@@ -169,6 +169,7 @@ def test_sgmv_shrink_tile_variants(r, h_in, lens):
     (2048, [1, 0, 3, 17, 1, 64, 5, 0, 130], None),
     (1160, [300, 2, 31, 257], None),             # 18 panels of 64 columns and one of 8
     (1024, [70, 1, 1, 600], (512, 384)),         # a column window of a wider y
+    (512, [288, 289, 545, 16], None),            # remainders that are merged into the other tiles, and one that is not
     (8, [5, 40], None),
 ])
 def test_sgmv_expand_transposed_b(dtype, r, h_out, lens, window):
