@@ -61,7 +61,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     const ShrinkGroup grp, const typename D::E* __restrict__ X, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int64_t layer_idx,
     int stages, float scale, int accumulate_into_v, int rows_per_tile, int kparts, int tile_slots,
-    float* __restrict__ partials) {
+    float* __restrict__ partials, int rotate) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   // The A tile stacks the A matrices of grp.count projections of rank r: row p * r + i is row i of
@@ -136,9 +136,20 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
       const E* Ap = proj == 0 ? A[0] : (proj == 1 ? A[1] : (proj == 2 ? A[2] : A[3]));
       asrc[j] = Ap + static_cast<int64_t>(arow) * h_in + k_begin + (((id & 15) ^ (row & 15)) << 3);
     }
+    // Where this tile starts its walk over the hidden dimension (it wraps round).  Workgroups that all walk from
+    // k = 0 ask for the same 256-byte column of rows a power-of-two-ish number of bytes apart at the same time,
+    // i.e. for the same few memory channels: x alone then streams at 4.0-5.3 TB/s for row lengths of 16, 28, 32
+    // or 56 KB where staggered walks reach 6.0-6.5 TB/s.  The tiles of one segment that run on one XCD stay
+    // within a few stages of each other, so that they still find the segment's A tiles in that XCD's L2.
+    // Tiles that read the same stack of A (one adapter, whatever the segment) keep the same start.
+    const unsigned who = static_cast<unsigned>(reinterpret_cast<uintptr_t>(A[0]) >> 12) * 2654435761u >> 20;
+    const int rot = rotate ? static_cast<int>((37u * (who * kXcds + blockIdx.x % kXcds) +
+                                               static_cast<unsigned>(rt.index) % 8u) % static_cast<unsigned>(nst))
+                           : 0;
     auto issue = [&](int st, int slot) {
       char* buf = lds + slot * kStageBytes;
-      const int k = st * kLdsKc;
+      const int sr = st + rot;
+      const int k = (sr >= nst ? sr - nst : sr) * kLdsKc;
 #pragma unroll
       for (int j = 0; j < kXLoads; ++j)
         __builtin_amdgcn_global_load_lds((const LORAX_GLOBAL void*)(xsrc[j] + k),
@@ -343,7 +354,8 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, grp, static_cast<const typename D::E*>(a.x),
                      a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages,
-                     a.scale, a.accumulate, rows_per_tile, kparts, static_cast<int>(tiles), a.partials);
+                     a.scale, a.accumulate, rows_per_tile, kparts, static_cast<int>(tiles), a.partials,
+                     tuning().shrink_no_rotate ? 0 : 1);
   e = hipGetLastError();
   if (e != hipSuccess || kparts == 1) return e;
   hipLaunchKernelGGL(sgmv_shrink_parts_kernel<D>, dim3(static_cast<unsigned>(tiles)), dim3(kLdsThreads), 0, stream, grp,

@@ -16,6 +16,7 @@ struct RowTile {
   int seg;      // segment (problem) index
   int row0;     // first row of the tile
   int row_end;  // one past the last row of the tile (<= end of segment)
+  int index;    // number of the tile inside its segment
 };
 
 // One chunk of 64 segments: lane `lane` holds the clamped bounds (s, e) of segment seg0 + lane.  If `tile`
@@ -53,6 +54,7 @@ __device__ __forceinline__ bool tile_in_chunk(int s, int e, int seg0, int rows_p
     const int s_f = __shfl(s, src, kWave);
     const int e_f = __shfl(e, src, kWave);
     out.seg = seg0 + src;
+    out.index = ti;
     if (MERGE) {
       const int nt_f = __shfl(nt, src, kWave);
       const int blocks = (e_f - s_f + 15) / 16;
