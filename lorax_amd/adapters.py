@@ -21,6 +21,7 @@ import torch
 from lorax_amd.sgmv import (
     BGMV_MAX_RANK,
     MAX_RANK_CUSTOM,
+    MIN_RANK_CUSTOM,
     get_tmp_tensors,
     orient_for_rank,
     pad_rank,
@@ -114,15 +115,17 @@ class LoraWeights(AdapterWeights):
         self._weights_b_t = torch.stack([w.transpose(0, 1).contiguous() for w in weights_b])  # [L, h_out, r]
         self._weights_a: Optional[torch.Tensor] = None
         self._weights_b: Optional[torch.Tensor] = None
+        self._rank_chunks = None
         self.adapter_config = adapter_config
 
     @property
     def weights_a(self) -> torch.Tensor:
         """The reference's prefill layout of A (orient_for_rank, punica.py:83-86)."""
         if self._weights_a is None:
-            # only below rank 16 do the two layouts disagree about A
+            # the layouts agree about A for the ranks of the reference's custom shrink (16 to 128) only
             a = self._weights_a_t
-            self._weights_a = a.transpose(1, 2).contiguous() if self._use_cutlass_shrink else a
+            same = MIN_RANK_CUSTOM <= self.lora_a_r <= MAX_RANK_CUSTOM
+            self._weights_a = a if same else a.transpose(1, 2).contiguous()
         return self._weights_a
 
     @property
@@ -135,6 +138,20 @@ class LoraWeights(AdapterWeights):
     @property
     def weights_a_t(self) -> torch.Tensor:
         return self._weights_a_t
+
+    def rank_chunks(self) -> List[Tuple[torch.Tensor, torch.Tensor, int]]:
+        """An adapter of a rank above what the kernels take (MAX_RANK_CUSTOM) as several adapters of kernel rank:
+        (x A^T) B = sum over chunks c of (x A_c^T) B_c with A_c the rows and B_c the columns [c * 128, ...) of the
+        stacks.  Returns [(A_c [L, r_c, h_in], B_c^T [L, h_out, r_c], r_c)], contiguous copies made on first use.
+        (The reference runs such adapters through its dense per-adapter loop, utils/layers.py:169-190.)"""
+        if self._rank_chunks is None:
+            step = MAX_RANK_CUSTOM
+            self._rank_chunks = [
+                (self._weights_a_t[:, c : c + step, :].contiguous(), self._weights_b_t[:, :, c : c + step].contiguous(),
+                 min(step, self.lora_a_r - c))
+                for c in range(0, self.lora_a_r, step)
+            ]
+        return self._rank_chunks
 
     @property
     def weights_b_t(self) -> torch.Tensor:
@@ -279,7 +296,7 @@ class BatchLoraWeights(BatchAdapterWeights):
     lora_a: Mapping  # adapter index -> A stack in the reference's prefill layout (built on access)
     lora_b: Mapping  # adapter index -> B stack [L, r, h_out] (built on access)
     adapter_index_configs: Dict[int, LoraConfig]
-    rank_data: Dict[int, RankSegments]
+    rank_data: Dict[object, RankSegments]  # rank -> group; (rank, chunk) -> group for ranks above 128
     use_sgmv: bool
     layer_name: str
     prefill_head_indices: Optional[torch.Tensor]
@@ -323,7 +340,8 @@ class BatchLoraWeights(BatchAdapterWeights):
         # adapter -> stack in the reference's prefill layout, read (and materialised) on access only
         lora_a = _LayoutView({seg_adapters[s]: loras[seg_adapters[s]] for s in covered}, "weights_a")
         lora_b = _LayoutView({seg_adapters[s]: loras[seg_adapters[s]] for s in covered}, "weights_b")
-        max_rank = max(loras[seg_adapters[s]].lora_a_r for s in covered)
+        # ranks above the kernels' limit are served as chunks of kernel rank, so decode stays on the BGMV tables
+        max_rank = min(max(loras[seg_adapters[s]].lora_a_r for s in covered), MAX_RANK_CUSTOM)
         use_sgmv = bool(prefill or max_rank > BGMV_MAX_RANK)
 
         # One pointer per segment; segments without weights hold a placeholder address that no
@@ -341,9 +359,16 @@ class BatchLoraWeights(BatchAdapterWeights):
 
         configs = {seg_adapters[s]: loras[seg_adapters[s]].adapter_config for s in covered}
 
-        by_rank: Dict[int, List[int]] = defaultdict(list)
+        # A rank group is keyed by its rank, as in the reference; chunk c of the adapters of a rank above 128 forms a
+        # group of its own under the key (rank, c), with the chunk's rank and the chunk stacks' addresses.
+        by_rank: Dict[object, List[int]] = defaultdict(list)
         for s in covered:
-            by_rank[loras[seg_adapters[s]].lora_a_r].append(s)
+            w = loras[seg_adapters[s]]
+            if w.lora_a_r <= MAX_RANK_CUSTOM:
+                by_rank[w.lora_a_r].append(s)
+            else:
+                for c in range(len(w.rank_chunks())):
+                    by_rank[(w.lora_a_r, c)].append(s)
 
         head_starts = head_ends = None
         if prefill_head_indices is not None:
@@ -360,8 +385,20 @@ class BatchLoraWeights(BatchAdapterWeights):
                     j += 1
 
         token_adapters = None if use_sgmv else meta.adapter_indices.tolist()
-        rank_data: Dict[int, RankSegments] = {}
-        for rank, segs in by_rank.items():
+        rank_data: Dict[object, RankSegments] = {}
+        for group_key, segs in by_rank.items():
+            chunk = group_key[1] if isinstance(group_key, tuple) else None
+            if chunk is None:
+                rank = group_key
+                group_a, group_b = a_addr, b_addr
+            else:  # addresses and rank of chunk `chunk` of every adapter of the group
+                rank = loras[seg_adapters[segs[0]]].rank_chunks()[chunk][2]
+                group_a, group_b = list(a_addr), list(b_addr)
+                for s in segs:
+                    a_c, b_c, _ = loras[seg_adapters[s]].rank_chunks()[chunk]
+                    group_a[s], group_b[s] = a_c.data_ptr(), b_c.data_ptr()
+            group_a_ptr = lora_a_t_ptr if chunk is None else torch.tensor(group_a, dtype=torch.int64, device=device)
+            group_b_ptr = lora_b_t_ptr if chunk is None else torch.tensor(group_b, dtype=torch.int64, device=device)
             if use_sgmv:
                 # the order of a group's segments is free: keep the segments of one adapter together, so that
                 # their tiles run back to back and share the adapter's weights in L2, adapters with the most
@@ -381,17 +418,20 @@ class BatchLoraWeights(BatchAdapterWeights):
                 slot: Dict[int, int] = {}
                 for pos, s in enumerate(segs):
                     slot.setdefault(seg_adapters[s], pos)
-                slots = [slot.get(a, -1) if (a in loras and loras[a].lora_a_r == rank) else -1 for a in token_adapters]
+                in_group = {seg_adapters[s] for s in segs}
+                slots = [slot.get(a, -1) if a in in_group else -1 for a in token_adapters]
                 token_slots = torch.tensor(slots, dtype=torch.int64, device=device)
-                records = build_bgmv_plan(slots, [a_addr[s] for s in segs], [b_addr[s] for s in segs])
+                records = build_bgmv_plan(slots, [group_a[s] for s in segs], [group_b[s] for s in segs])
                 plan = torch.tensor(records, dtype=torch.int64, device=device).reshape(-1, BGMV_PLAN_WORDS)
-            if use_sgmv:
+            if use_sgmv and chunk is None:
                 # the reference's prefill tables, built (with the weight copies behind them) on first access
                 ref_a = (lambda segs=segs: table("weights_a")[segs])
                 ref_b = (lambda segs=segs: table("weights_b")[segs])
+            elif use_sgmv:
+                ref_a = ref_b = None  # rank chunks exist in the resident layouts only
             else:
-                ref_a, ref_b = lora_a_t_ptr[segs], lora_b_t_ptr[segs]
-            rank_data[rank] = RankSegments(
+                ref_a, ref_b = group_a_ptr[segs], group_b_ptr[segs]
+            rank_data[group_key] = RankSegments(
                 rank=rank,
                 lora_a_ptr=ref_a,
                 lora_b_ptr=ref_b,
@@ -401,9 +441,9 @@ class BatchLoraWeights(BatchAdapterWeights):
                 segment_ends=ends,
                 indices=token_slots,
                 plan=plan,
-                lora_a_t_ptr=lora_a_t_ptr[segs] if use_sgmv else None,
-                lora_b_t_ptr=lora_b_t_ptr[segs] if use_sgmv else None,
-                segments_key=(tuple(segs), head_starts is not None) if use_sgmv else None,
+                lora_a_t_ptr=group_a_ptr[segs] if use_sgmv else None,
+                lora_b_t_ptr=group_b_ptr[segs] if use_sgmv else None,
+                segments_key=(tuple(segs), head_starts is not None, chunk) if use_sgmv else None,
             )
 
         return cls(
@@ -444,7 +484,7 @@ class LayerAdapterWeights:
     def lora_entries(self):
         """(adapter, address of the [L, r, h_in] stack, address of the [L, h_out, r] stack, rank) of every LoRA
         adapter of the layer type, sorted by adapter, as a numpy array of _native.ENTRY_DTYPE; None if an adapter
-        of another kind is loaded.  Rebuilt only when adapters come or go."""
+        of another kind, or of a rank above the kernels' 128, is loaded.  Rebuilt only when adapters come or go."""
         if self._lora_entries is None:
             import numpy as np
 
@@ -455,6 +495,8 @@ class LayerAdapterWeights:
                 w = _unwrap(self.adapter_weights[idx])
                 if not isinstance(w, LoraWeights) or w.get_batch_types() != [BatchLoraWeights]:
                     return None
+                if w.lora_a_r > MAX_RANK_CUSTOM:
+                    return None  # served in rank chunks, which the per-layer-type Python path builds
                 rows.append((idx, w.weights_a_t.data_ptr(), w.weights_b_t.data_ptr(), w.lora_a_r, 0))
             self._lora_entries = np.array(rows, dtype=_native.ENTRY_DTYPE)
         return self._lora_entries

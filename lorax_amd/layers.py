@@ -86,7 +86,7 @@ class LoraLinear(nn.Module):
         """Adds the LoRA deltas of several projections that share `input`; projection `name` owns the
         columns [start, end) of `result`."""
         tensor_parallel = self.process_group.size() > 1
-        decode_jobs = defaultdict(list)  # rank -> [(rank_segments, start, width)]
+        decode_jobs = defaultdict(list)  # (wave, rank) -> [(rank_segments, start, width)]
         stacked_jobs = []  # (lora_a_stack, lora_b_stack, start, width) of projections served by stacked weights
         prefill_jobs = defaultdict(list)  # (rank, segment tables) -> [(rank_segments, start, width)]
         for name, start, end in slices:
@@ -107,11 +107,14 @@ class LoraLinear(nn.Module):
                 stacked_jobs.append((lora_a_weights, lora_b_weights, start, end - start))
                 continue
             sliced = end - start != result.shape[1]
-            for r, rs in data.rank_data.items():
+            for group_key, rs in data.rank_data.items():
+                r = rs.rank  # the kernels' rank: that of the group, or of its chunk of a rank above 128
                 if not data.use_sgmv:
                     if rs.lora_a_ptr is None or rs.lora_b_ptr is None:
                         continue
-                    decode_jobs[r].append((rs, start, end - start))
+                    # the chunks of one adapter update the same elements of the result: one launch per chunk number
+                    wave = group_key[1] if isinstance(group_key, tuple) else 0
+                    decode_jobs[(wave, r)].append((rs, start, end - start))
                     continue
                 # Prefill reads the resident stacks ([L, r, h_in] and [L, h_out, r], the ones decode uses);
                 # the reference's prefill layouts are only touched for shapes the resident-layout shrink
@@ -125,6 +128,11 @@ class LoraLinear(nn.Module):
                         self.layer_id, r, zero_fill=tensor_parallel,
                     )
                 else:
+                    if rs.lora_a_ptr is None:
+                        raise RuntimeError(
+                            f"rank chunk of {r} over h_in={input.size(1)}: no kernel takes this shape from the resident "
+                            "layout, and rank chunks have no other"
+                        )
                     v = lora_a_sgmv_cutlass(
                         input, rs.tmp_shrink, rs.lora_a_ptr, rs.segment_starts, rs.segment_ends, self.layer_id, r
                     )
@@ -182,13 +190,23 @@ class LoraLinear(nn.Module):
         # expand run in one launch per rank and v never leaves the chip.  Otherwise all rank groups of all
         # projections go out together: one shrink launch and one expand launch per 16 problems, whatever the
         # mix of ranks (the reference issues a pair of launches per projection and rank, layers.py:146-164).
-        jobs = [(r, rs, start, width) for r, rank_jobs in decode_jobs.items() for rs, start, width in rank_jobs]
+        waves = sorted({wave for wave, _ in decode_jobs})
+        if len(waves) > 1:
+            for wave in waves:
+                self._decode(result, input, {k: v for k, v in decode_jobs.items() if k[0] == wave}, tensor_parallel)
+            return result
+        return self._decode(result, input, decode_jobs, tensor_parallel)
+
+    def _decode(self, result, input, decode_jobs, tensor_parallel):
+        """The decode launches of forward_layer_types for jobs that touch disjoint elements of `result`:
+        decode_jobs maps (wave, rank) to [(rank_segments, start, width)]."""
+        jobs = [(r, rs, start, width) for (_, r), rank_jobs in decode_jobs.items() for rs, start, width in rank_jobs]
         all_fused = bool(jobs) and not tensor_parallel and all(
             rs.plan is not None and _native.bgmv_lora_fits(r, input.size(1), width) for r, rs, _, width in jobs
         )
         if all_fused:
             step = _native.MAX_FUSED_BGMV_PROBLEMS
-            for r in decode_jobs:
+            for r in sorted({r for _, r in decode_jobs}):
                 single = [j for j in jobs if j[0] == r]
                 for i in range(0, len(single), step):
                     _native.bgmv_lora_multi(

@@ -194,3 +194,56 @@ def test_lm_head_with_a_large_vocabulary(prefill):
     untouched = torch.tensor([a not in ranks for a in request_adapters])
     assert torch.equal(logits.cpu()[untouched], y0[untouched])
     assert torch.count_nonzero(logits.cpu()[~untouched] != y0[~untouched]) > 0
+
+
+@pytest.mark.parametrize("mode,lens", [
+    ("decode", [1] * 12),
+    ("prefill", [40, 3, 9, 1, 17, 5, 30, 2, 8, 1, 6, 11]),          # a short batch
+    ("prefill", [300, 3, 90, 1, 170, 50, 30, 2, 80, 1, 60, 110]),   # past the streaming kernels' range
+])
+def test_ranks_above_the_kernel_limit_run_as_rank_chunks(mode, lens):
+    """Adapters of rank 192 and 256 next to one of rank 16 and requests without adapter, on a fused q/k/v
+    projection: the kernels take ranks up to 128, so such an adapter is served as chunks of its rank (128 + 64,
+    128 + 128), each a rank group of its own.  The oracle multiplies with the whole rank at once."""
+    from lorax_amd.adapters import AdapterBatchData, LayerAdapterWeights, LoraConfig, LoraWeights
+    from lorax_amd.synthetic import make_meta
+
+    prefill = mode == "prefill"
+    dtype, hidden, layers, layer_id = torch.bfloat16, 1024, 2, 1
+    names, sizes = ["q_proj", "k_proj", "v_proj"], [1024, 256, 256]
+    gen = torch.Generator().manual_seed(len(lens) + sum(lens))
+    request_adapters = [0, 1, 2, 9, 1, 0, 2, 2, 9, 0, 1, 1]      # 9 has no weights
+    ranks = {0: 192, 1: 256, 2: 16}
+    tokens = [a for a, n in zip(request_adapters, lens) for _ in range(n)]
+    meta = make_meta(tokens, torch.device(DEV))
+    weights = {}
+    for name, size in zip(names, sizes):
+        layer = LayerAdapterWeights()
+        for a, r in ranks.items():
+            wa = (torch.randn((layers, hidden, r), generator=gen) * 0.05).to(dtype).to(DEV)
+            wb = (torch.randn((layers, r, size), generator=gen) * 0.05).to(dtype).to(DEV)
+            layer.add_adapter(a, LoraWeights(list(wa.unbind(0)), list(wb.unbind(0)), LoraConfig(r=r)))
+        weights[name] = layer
+    batch = AdapterBatchData.from_meta(meta, weights, prefill=prefill)
+    groups = batch.data["q_proj"][LORA].rank_data
+    assert sorted(map(str, groups)) == sorted(map(str, [16, (192, 0), (192, 1), (256, 0), (256, 1)]))
+    assert sorted(rs.rank for rs in groups.values()) == [16, 64, 128, 128, 128]
+    assert batch.data["q_proj"][LORA].use_sgmv == prefill
+
+    T = len(tokens)
+    x = torch.randn((T, hidden), generator=gen).to(dtype)
+    y0 = (torch.randn((T, sum(sizes)), generator=gen) * 0.25).to(dtype)
+    proj = TensorParallelMultiAdapterLinear.load(ZeroBase(y0.to(DEV)), layer_id, names, sizes)
+    out = proj(x.to(DEV), batch)
+    torch.cuda.synchronize()
+    ref, off, idx = y0.clone(), 0, torch.tensor(tokens)
+    for name, size in zip(names, sizes):
+        lora_a = {a: lw.weights_a.cpu() for a, lw in weights[name].adapter_weights.items()}
+        lora_b = {a: lw.weights_b.cpu() for a, lw in weights[name].adapter_weights.items()}
+        O.fallback_layer_type(ref, x, idx, set(tokens), lora_a, lora_b, layer_id, off, off + size)
+        off += size
+    delta = (ref.float() - y0.float()).to(dtype)
+    # a chunked adapter's update reaches y in two roundings (one per chunk) instead of one
+    assert_close(out, ref, f"rank chunks, {mode}", rounded=[delta, delta])
+    untouched = torch.tensor([a not in ranks for a in tokens])
+    assert torch.equal(out.cpu()[untouched], y0[untouched])

@@ -21,6 +21,7 @@ from lorax_amd.adapters import (
     LoraWeights,
     get_scaling_factor,
 )
+from lorax_amd.layers import SingleProcessGroup
 from lorax_amd.segments import SegmentConcatBuilder, find_segments
 from oracle import lora_oracle as O
 
@@ -218,6 +219,47 @@ def test_lora_weights_layouts_stay_resident():
             assert ptrs == (w.weights_a.data_ptr(), w.weights_b.data_ptr(), w.weights_a_t.data_ptr(),
                             w.weights_b_t.data_ptr())
         assert torch.equal(w.weights_a_t[1], a[1].t()) and torch.equal(w.weights_b_t[2], b[2].t())
+
+
+def test_ranks_above_128_become_rank_chunks():
+    """An adapter of rank 192 is split into chunks of kernel rank (128 + 64); every chunk is a rank group of its
+    own whose tables hold the chunk stacks' addresses.  The reference's layouts of the whole stack stay available
+    ([L, h_in, r] for A above rank 128, orient_for_rank, punica.py:83-86)."""
+    h_in, h_out, r = 64, 48, 192
+    a = [torch.randn(h_in, r) for _ in range(2)]
+    b = [torch.randn(r, h_out) for _ in range(2)]
+    big = LoraWeights(a, b, LoraConfig(r=r))
+    small = LoraWeights([torch.randn(h_in, 16)] * 2, [torch.randn(16, h_out)] * 2, LoraConfig(r=16))
+    assert big.weights_a.shape == (2, h_in, r) and big.weights_b.shape == (2, r, h_out)
+    chunks = big.rank_chunks()
+    assert [c[2] for c in chunks] == [128, 64] and big.rank_chunks() is chunks
+    assert torch.equal(chunks[1][0][1], a[1].t()[128:]) and torch.equal(chunks[1][1][0], b[0].t()[:, 128:])
+    x = torch.randn(5, h_in)
+    whole = x @ a[0] @ b[0]
+    parts = sum((x @ ca[0].t()) @ cb[0].t() for ca, cb, _ in chunks)
+    assert torch.allclose(parts, whole, atol=1e-3)
+
+    layer = LayerAdapterWeights()
+    layer.add_adapter(0, big)
+    layer.add_adapter(1, small)
+    assert layer.lora_entries() is None  # the native table builder leaves such a layer type to the Python path
+    tokens = [0, 0, 1, 0, 1]
+    for prefill in (False, True):
+        meta = _meta(tokens)
+        data = layer.get_data(meta, "q_proj", prefill, None)[LORA]
+        assert data.use_sgmv == prefill and data.can_vectorize(SingleProcessGroup())
+        assert set(data.rank_data) == {16, (192, 0), (192, 1)}
+        for c, (ca, cb, rc) in enumerate(chunks):
+            rs = data.rank_data[(192, c)]
+            assert rs.rank == rc
+            a_tab = rs.lora_a_t_ptr if prefill else rs.lora_a_ptr
+            b_tab = rs.lora_b_t_ptr if prefill else rs.lora_b_ptr
+            assert set(a_tab.tolist()) == {ca.data_ptr()} and set(b_tab.tolist()) == {cb.data_ptr()}
+            if prefill:
+                assert rs.lora_a_ptr is None and rs.segment_starts.tolist() == [0, 3] and rs.segment_ends.tolist() == [2, 4]
+            else:
+                assert rs.indices.tolist() == [0, 0, -1, 0, -1]
+                assert sorted(rec[0] for rec in rs.plan.tolist()) == [3]
 
 
 def test_from_peft_folds_scale_and_pads():
