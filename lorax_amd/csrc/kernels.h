@@ -132,11 +132,11 @@ hipError_t launch_sgmv_lora_rows(const SgmvLoraArgs& a, hipStream_t stream);
 struct Tuning {
   int bgmv_lora_blocks;  // LORAX_BGMV_LORA_BLOCKS: expand blocks per workgroup of the single-launch BGMV (1, 2, 4)
   int bgmv_shrink_rows;  // LORAX_BGMV_SHRINK_ROWS: rows of A per workgroup of the BGMV shrink (2, 4, 8)
-  int shrink_ksplit;     // LORAX_SHRINK_KSPLIT: K splits across workgroups of the register-operand SGMV shrink
+  int shrink_ksplit;     // LORAX_SHRINK_KSPLIT: K splits (parts) across workgroups of the SGMV shrinks
   int shrink_mb;         // LORAX_SHRINK_MB: 16-row blocks per row tile of the SGMV shrink (1, 2, 4)
   int shrink_waves;      // LORAX_SHRINK_WAVES: waves per workgroup of the register-operand SGMV shrink
   int expand_rows;       // LORAX_EXPAND_ROWS: rows per tile of the SGMV expand
-  int shrink_no_rotate;  // LORAX_SHRINK_NO_ROTATE: register-operand SGMV shrink without the K rotation per tile
+  int shrink_no_rotate;  // LORAX_SHRINK_NO_ROTATE: SGMV shrinks whose tiles all walk the hidden dimension from k = 0
   int shrink_lds;  // LORAX_SHRINK_LDS: 1 = always take the LDS-staged shrink where it applies, -1 = never
   int shrink_lds_kb;  // LORAX_SHRINK_LDS_KB: LDS budget of the staged shrink's buffers
   int bgmv_expand_cols;  // LORAX_BGMV_EXPAND_COLS: columns per lane group of the BGMV expand (4, 8, 16)
