@@ -81,8 +81,10 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
   // stage for all blocks of the tile and the partial sums are added through LDS at the end (every
   // staged byte is read from LDS once).  Otherwise: waves as WM x WN over the (row block, rank
   // block) grid, each with its own output blocks and all k.
-  constexpr int WN = KSPLIT ? 1 : ((NB % 2 == 0) ? 2 : 1);
+  // (three row blocks - 48-row tiles - only divide as 1 x 4, which needs the rank blocks to be a multiple of 4)
+  constexpr int WN = KSPLIT ? 1 : (MBLK % 2 != 0 ? 4 : ((NB % 2 == 0) ? 2 : 1));
   constexpr int WM = KSPLIT ? 1 : 4 / WN;
+  static_assert(KSPLIT || NB % WN == 0, "rank blocks must divide among the waves");
   static_assert(MBLK % WM == 0, "row blocks must divide among the waves");
   // KSPLIT: the partial sums (4 * MBLK * NB KB) go where the stage buffers are; the launcher sizes the LDS for it
   constexpr int MPW = MBLK / WM;  // row blocks per wave
@@ -286,7 +288,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_parts_kernel(
 // Host side
 // ---------------------------------------------------------------------------------
 template <typename D, int NB, int MBLK, bool KSPLIT>
-static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
+static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_rows = 0) {
   constexpr int kStageBytes = (MBLK + NB) * 16 * kLdsRowBytes;
   constexpr int kRedBytes = KSPLIT ? 4 * MBLK * NB * 1024 : 0;  // partial sums of the four waves at the end of a tile
   static_assert(kRedBytes <= kLdsMaxBytes, "partial sums must fit in LDS");
@@ -294,12 +296,20 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream) {
   // are fewer than the 256 CUs the tiles are lowered (in steps of 16 rows) until they are about as many.  The
   // host knows the rows and the number of segments, not their lengths: ceil(T / M) + segments bounds the count.
   int rows_per_tile = MBLK * 16;
-  if (tuning().shrink_rows <= 0) {
+  if (fixed_rows > 0) {
+    rows_per_tile = fixed_rows;
+  } else if (tuning().shrink_rows <= 0) {
     while (rows_per_tile > 16 &&
            (a.num_tokens + rows_per_tile - 17) / (rows_per_tile - 16) + a.num_segments <= 256)
       rows_per_tile -= 16;
   } else if (tuning().shrink_rows < rows_per_tile) {
     rows_per_tile = (tuning().shrink_rows + 15) / 16 * 16;
+  }
+  // Tiles of 48 rows in buffers of 48: the fourth row block of 64-row buffers would be staged (re-reading the
+  // tile's last row) and multiplied for nothing.
+  if constexpr (MBLK == 4 && (KSPLIT || NB % 4 == 0)) {
+    if (rows_per_tile == 48 && fixed_rows == 0 && tuning().shrink_mb == 0)
+      return launch_lds_m<D, NB, 3, KSPLIT>(a, stream, 48);
   }
   const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
   // K parts: a workgroup streams its tile's x and A at about 50 GB/s whatever the launch, so a launch of a
