@@ -321,9 +321,126 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
   }
 }
 
-template <typename D, int CP, int U>
+// The same with y moved in whole 16-byte pieces (every problem's y rows 16-byte aligned: y_offset and y_stride
+// multiples of 8).  Above, a lane reads and writes single elements of y, so a wave spends U * NT load and as many
+// store instructions of 32-128 useful bytes on y, more instructions than it spends on B^T.  Here the sums change
+// lanes through a piece of LDS private to the wave: per step the wave's lane groups hold 64 / CP ADJACENT columns,
+// so once all steps' sums are written as [token][step][column], item i is 8 (or 4, at 16 lanes per column) adjacent
+// columns of one token and step, and lane i % 64 owns it: one 16-byte load of the old y, issued in front with the
+// loads of B^T, and one 16-byte store.  Same sums, same roundings: the result equals the scalar path's bit for bit.
+template <typename D, int CP, int U, int NT>
+__device__ __forceinline__ void bgmv_expand_body_vec(typename D::E* __restrict__ Y,
+                                                     const typename D::E* __restrict__ V,
+                                                     const typename D::E* __restrict__ B,
+                                                     const int (&toks)[kGroup], int r, int h_out,
+                                                     int col0, int64_t y_offset, int64_t y_stride,
+                                                     float scale, bool accumulate_into_y, float* wave_sums) {
+  using vec8 = typename D::vec8;
+  using E = typename D::E;
+  constexpr int GPW = kWave / CP;           // adjacent columns per step of one wave
+  constexpr int VC = GPW >= 8 ? 8 : 4;      // columns per y access
+  constexpr int PIECES = GPW / VC;          // y accesses per token and step
+  constexpr int ITEMS = NT * U * PIECES;
+  constexpr int KI = (ITEMS + kWave - 1) / kWave;
+  typedef E vecy __attribute__((ext_vector_type(VC)));
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int part = tid % CP;
+  const int ql = lane / CP;  // the lane group's column inside the wave's run
+  const bool has_k = part * 8 < r;
+
+  vec8 vv[NT];
+#pragma unroll
+  for (int g = 0; g < NT; ++g) {
+    vv[g] = zero8<D>();
+    if (has_k) vv[g] = load8<D>(V + static_cast<int64_t>(toks[g]) * r + part * 8);
+  }
+  vec8 wv[U];
+  // A wave's U steps cover U * GPW adjacent columns (the scalar path deals the steps kCols apart): the B^T rows of
+  // one step are as contiguous as there, and the wave's y accesses for one token are one run of whole cache lines.
+  const int colbase = col0 + wave * U * GPW + ql;  // the lane group's column of step u is colbase + u * GPW
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int c = colbase + u * GPW;
+    wv[u] = zero8<D>();
+    if (has_k && c < h_out) wv[u] = load8<D>(B + static_cast<int64_t>(c) * r + part * 8);
+  }
+  // this lane's items: i = (token * U + step) * PIECES + piece
+  vecy yold[KI];
+  E* yp[KI];
+  bool live[KI];
+#pragma unroll
+  for (int k = 0; k < KI; ++k) {
+    const int i = lane + k * kWave;
+    const int piece = i % PIECES;
+    const int u = (i / PIECES) % U;
+    const int g = i / (PIECES * U);
+    const int c = col0 + (wave * U + u) * GPW + piece * VC;
+    live[k] = i < ITEMS && c < h_out;  // h_out is a multiple of 8: a piece is inside or outside as a whole
+    // (the values are made opaque so that the optimiser keeps a select chain instead of turning toks[] into an
+    // array in memory indexed by the lane's g)
+    int tok = toks[0];
+#pragma unroll
+    for (int q = 1; q < NT; ++q) {
+      int t = toks[q];
+      asm volatile("" : "+v"(t));
+      tok = g == q ? t : tok;
+    }
+    yp[k] = Y + static_cast<int64_t>(tok) * y_stride + y_offset + c;
+#pragma unroll
+    for (int e = 0; e < VC; ++e) yold[k][e] = static_cast<E>(0.f);
+    if (live[k] && accumulate_into_y) yold[k] = *(const LORAX_GLOBAL vecy*)(yp[k]);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    float s[NT];
+#pragma unroll
+    for (int g = 0; g < NT; ++g) s[g] = dot8<D>(wv[u], vv[g], 0.f);
+#pragma unroll
+    for (int m = CP / 2; m >= 1; m >>= 1)
+#pragma unroll
+      for (int g = 0; g < NT; ++g) s[g] += __shfl_xor(s[g], m, kWave);
+    if (part == u % CP) {
+#pragma unroll
+      for (int g = 0; g < NT; ++g) wave_sums[(g * U + u) * GPW + ql] = s[g] * scale;
+    }
+  }
+  // Writer and reader are lanes of one wave and a wave's LDS accesses execute in order: only the compiler has
+  // to be kept from moving the reads up.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int k = 0; k < KI; ++k) {
+    if (live[k]) {
+      const float* d = wave_sums + (lane + k * kWave) * VC;
+      vecy out;
+#pragma unroll
+      for (int e = 0; e < VC; e += 4) {
+        const f32x4 q = *reinterpret_cast<const f32x4*>(d + e);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) out[e + t] = accumulate<D>(yold[k][e + t], q[t]);
+      }
+      *(LORAX_GLOBAL vecy*)(yp[k]) = out;
+    }
+  }
+}
+
+template <typename D, int CP, int U, int NT, bool VY>
+__device__ __forceinline__ void bgmv_expand_tokens(typename D::E* Y, const typename D::E* V, const typename D::E* B,
+                                                   const int (&toks)[kGroup], int r, int h_out, int col0,
+                                                   int64_t y_offset, int64_t y_stride, float scale, bool acc_y,
+                                                   float* wave_sums) {
+  if constexpr (VY)
+    bgmv_expand_body_vec<D, CP, U, NT>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale, acc_y, wave_sums);
+  else
+    bgmv_expand_body<D, CP, U, NT>(Y, V, B, toks, r, h_out, col0, y_offset, y_stride, scale, acc_y);
+}
+
+template <typename D, int CP, int U, bool VY>
 __device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const BatchSlot& slot, int num_tokens,
-                                                    int64_t layer_idx, float scale, bool acc_y) {
+                                                    int64_t layer_idx, float scale, bool acc_y, float* wave_sums) {
   using E = typename D::E;
   const int h_out = P.width;
   const int r = P.narrow;
@@ -337,16 +454,16 @@ __device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const 
   const E* V = static_cast<const E*>(P.x);
   switch (n) {
     case 1:
-      bgmv_expand_body<D, CP, U, 1>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
+      bgmv_expand_tokens<D, CP, U, 1, VY>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y, wave_sums);
       break;
     case 2:
-      bgmv_expand_body<D, CP, U, 2>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
+      bgmv_expand_tokens<D, CP, U, 2, VY>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y, wave_sums);
       break;
     case 3:
-      bgmv_expand_body<D, CP, U, 3>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
+      bgmv_expand_tokens<D, CP, U, 3, VY>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y, wave_sums);
       break;
     default:
-      bgmv_expand_body<D, CP, U, 4>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y);
+      bgmv_expand_tokens<D, CP, U, 4, VY>(Y, V, B, toks, r, h_out, col0, P.y_offset, P.y_stride, scale, acc_y, wave_sums);
       break;
   }
 }
@@ -365,28 +482,34 @@ __host__ __device__ __forceinline__ int expand_lanes_per_column(int r) {
 }
 
 // One launch serves problems of different ranks: the workgroup picks the body for its problem's rank.
-template <typename D, int U>
+// VY: y moves in 16-byte pieces (bgmv_expand_body_vec); each wave has kGroup * U * 64 floats of LDS for its sums
+// (one lane per column, the widest case; with 4 and more lanes per column the steps double and the columns per
+// step shrink by more).
+template <typename D, int U, bool VY>
 __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBatch batch, int count,
                                                                    int num_tokens, int64_t layer_idx, float scale,
                                                                    int accumulate_into_y) {
+  constexpr int kWaveSums = kGroup * U * kWave;
+  __shared__ __attribute__((aligned(16))) float sums[VY ? (kBgmvThreads / kWave) * kWaveSums : 4];
+  float* wave_sums = sums + (VY ? (threadIdx.x / kWave) * kWaveSums : 0);
   const bool acc_y = accumulate_into_y != 0;
   const BatchSlot vb = batch_slot(batch, count);
   const BgmvProblem& P = batch.p[vb.problem];
   switch (expand_lanes_per_column(P.narrow)) {
     case 1:
-      bgmv_expand_problem<D, 1, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
+      bgmv_expand_problem<D, 1, U, VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
       break;
     case 2:
-      bgmv_expand_problem<D, 2, U>(P, vb, num_tokens, layer_idx, scale, acc_y);
+      bgmv_expand_problem<D, 2, U, VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
       break;
     case 4:
-      bgmv_expand_problem<D, 4, expand_steps(4, U)>(P, vb, num_tokens, layer_idx, scale, acc_y);
+      bgmv_expand_problem<D, 4, expand_steps(4, U), VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
       break;
     case 8:
-      bgmv_expand_problem<D, 8, expand_steps(8, U)>(P, vb, num_tokens, layer_idx, scale, acc_y);
+      bgmv_expand_problem<D, 8, expand_steps(8, U), VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
       break;
     default:
-      bgmv_expand_problem<D, 16, expand_steps(16, U)>(P, vb, num_tokens, layer_idx, scale, acc_y);
+      bgmv_expand_problem<D, 16, expand_steps(16, U), VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
       break;
   }
 }
@@ -838,8 +961,18 @@ static hipError_t launch_expand_u(BgmvArgs a, hipStream_t stream) {
   });
   if (total == 0) return hipSuccess;
   if (total >= INT32_MAX) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((bgmv_expand_kernel<D, U>), dim3(static_cast<unsigned>(total)), dim3(kBgmvThreads), 0, stream,
-                     a.batch, a.count, static_cast<int>(a.num_tokens), a.layer_idx, a.scale, a.accumulate);
+  // 16-byte y accesses need every problem's rows 16-byte aligned (the widths are multiples of 8)
+  bool vec_y = !tuning().bgmv_scalar_y;
+  for (int i = 0; i < a.count; ++i) {
+    const BgmvProblem& p = a.batch.p[i];
+    vec_y = vec_y && p.y_stride % 8 == 0 && p.y_offset % 8 == 0 && reinterpret_cast<uintptr_t>(p.y) % 16 == 0;
+  }
+  if (vec_y)
+    hipLaunchKernelGGL((bgmv_expand_kernel<D, U, true>), dim3(static_cast<unsigned>(total)), dim3(kBgmvThreads), 0,
+                       stream, a.batch, a.count, static_cast<int>(a.num_tokens), a.layer_idx, a.scale, a.accumulate);
+  else
+    hipLaunchKernelGGL((bgmv_expand_kernel<D, U, false>), dim3(static_cast<unsigned>(total)), dim3(kBgmvThreads), 0,
+                       stream, a.batch, a.count, static_cast<int>(a.num_tokens), a.layer_idx, a.scale, a.accumulate);
   return hipGetLastError();
 }
 

@@ -86,7 +86,7 @@ const Tuning& tuning() {
 #else
   static const Tuning t = {env_int("LORAX_BGMV_LORA_BLOCKS"), env_int("LORAX_BGMV_SHRINK_ROWS"), env_int("LORAX_SHRINK_KSPLIT"),
                            env_int("LORAX_SHRINK_MB"), env_int("LORAX_SHRINK_WAVES"), env_int("LORAX_EXPAND_ROWS"),
-                           env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB"), env_int("LORAX_BGMV_EXPAND_COLS"), env_int("LORAX_EXPAND_PANELS"), env_int("LORAX_BGMV_NO_RUNS"), env_int("LORAX_BGMV_NO_BALANCE"), env_int("LORAX_SHRINK_ROWS_MAX"), env_int("LORAX_SHRINK_ROWS")};
+                           env_int("LORAX_SHRINK_NO_ROTATE"), env_int("LORAX_SHRINK_LDS"), env_int("LORAX_SHRINK_LDS_KB"), env_int("LORAX_BGMV_EXPAND_COLS"), env_int("LORAX_EXPAND_PANELS"), env_int("LORAX_BGMV_NO_RUNS"), env_int("LORAX_BGMV_NO_BALANCE"), env_int("LORAX_SHRINK_ROWS_MAX"), env_int("LORAX_SHRINK_ROWS"), env_int("LORAX_BGMV_SCALAR_Y")};
 #endif
   return t;
 }

@@ -145,6 +145,7 @@ struct Tuning {
   int bgmv_no_balance;  // LORAX_BGMV_NO_BALANCE: plain workgroup numbering in the single-launch BGMV
   int shrink_rows_max;  // LORAX_SHRINK_ROWS_MAX: largest token count served by the streaming SGMV shrink (-1 = never)
   int shrink_rows;      // LORAX_SHRINK_ROWS: rows per tile of the LDS-staged SGMV shrink (below its buffers' height)
+  int bgmv_scalar_y;    // LORAX_BGMV_SCALAR_Y: BGMV expand that moves y element by element even where rows are aligned
 };
 const Tuning& tuning();
 

@@ -140,6 +140,34 @@ def test_bgmv_column_window_of_fused_output():
     assert_close(y, y_ref, "fused q/k/v output")
 
 
+@pytest.mark.parametrize("r", [8, 16, 24, 32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_bgmv_expand_vector_and_scalar_y_paths_agree_bit_for_bit(dtype, r):
+    """A y whose rows are 16-byte aligned moves in 16-byte pieces, any other element by element: same sums,
+    same roundings, so the same bits.  The second window starts 4 columns into rows of a pitch that is no
+    multiple of 8.  Chunks of 1 to 4 tokens per adapter, a last column block that is not full."""
+    print(f"case dtype={dtype} r={r}", flush=True)
+    T, h_out, n = 45, 2248, 7
+    gen = torch.Generator().manual_seed(500 + r)
+    wb_t = _stacks(n, 2, h_out, r, gen, dtype)
+    v = randn((T, r), 1.0, gen, dtype, DEV)
+    idx = _indices(T, n, gen)
+    idx[:9] = 0  # an adapter with more than two chunks
+    y0 = randn((T, h_out), 0.5, gen, dtype, DEV)
+    ya = y0.clone()
+    sgmv.add_lora_b_bgmv(ya, v, ptr_table(wb_t, DEV), idx.to(DEV), 1)
+    wide = torch.zeros((T, h_out + 12), dtype=dtype, device=DEV)
+    wide[:, 4:4 + h_out] = y0
+    sgmv.add_lora_b_bgmv_slice(wide, v, ptr_table(wb_t, DEV), idx.to(DEV), 1, 4, h_out)
+    torch.cuda.synchronize()
+    assert torch.equal(ya, wide[:, 4:4 + h_out])
+    assert torch.count_nonzero(wide[:, :4]) == 0 and torch.count_nonzero(wide[:, 4 + h_out:]) == 0
+    y_ref = y0.cpu().clone()
+    O.bgmv_ref(y_ref, v.cpu(), [w.cpu() for w in wb_t], idx.tolist(), 1)
+    assert_close(ya, y_ref, "expand output y")
+    assert torch.equal(ya.cpu()[idx < 0], y0.cpu()[idx < 0])
+
+
 def test_bgmv_under_graph_capture_replays_identically():
     dtype, T, h_in, h_out, r, n = torch.bfloat16, 64, 4096, 4096, 32, 9
     gen = torch.Generator().manual_seed(3)
