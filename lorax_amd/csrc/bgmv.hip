@@ -309,9 +309,7 @@ __device__ __forceinline__ void bgmv_expand_body(typename D::E* __restrict__ Y,
 #pragma unroll
     for (int g = 0; g < NT; ++g) s[g] = dot8<D>(wv[u], vv[g], 0.f);
 #pragma unroll
-    for (int m = CP / 2; m >= 1; m >>= 1)
-#pragma unroll
-      for (int g = 0; g < NT; ++g) s[g] += __shfl_xor(s[g], m, kWave);
+    for (int g = 0; g < NT; ++g) s[g] = group_sum<CP>(s[g]);
     const int c = colbase + u * kCols;
     if (part == u % CP && c < h_out) {
 #pragma unroll
@@ -398,9 +396,7 @@ __device__ __forceinline__ void bgmv_expand_body_vec(typename D::E* __restrict__
 #pragma unroll
     for (int g = 0; g < NT; ++g) s[g] = dot8<D>(wv[u], vv[g], 0.f);
 #pragma unroll
-    for (int m = CP / 2; m >= 1; m >>= 1)
-#pragma unroll
-      for (int g = 0; g < NT; ++g) s[g] += __shfl_xor(s[g], m, kWave);
+    for (int g = 0; g < NT; ++g) s[g] = group_sum<CP>(s[g]);
     if (part == u % CP) {
 #pragma unroll
       for (int g = 0; g < NT; ++g) wave_sums[(g * U + u) * GPW + ql] = s[g] * scale;
@@ -657,9 +653,7 @@ __device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
 #pragma unroll
       for (int g = 0; g < NT; ++g) s[g] = dot8<D>(w[u], vv[g], 0.f);
 #pragma unroll
-      for (int m = CP / 2; m >= 1; m >>= 1)
-#pragma unroll
-        for (int g = 0; g < NT; ++g) s[g] += __shfl_xor(s[g], m, kWave);
+      for (int g = 0; g < NT; ++g) s[g] = group_sum<CP>(s[g]);
       const int col = column(blk, u);
       if (part == 0 && col < col_end) {
 #pragma unroll
@@ -676,11 +670,9 @@ __device__ __forceinline__ void bgmv_lora_body(typename D::E* __restrict__ Y,
 #pragma unroll
         for (int g = 0; g < NT; ++g) s[u][g] = dot8<D>(wv[blk][u], vv[g], 0.f);
 #pragma unroll
-      for (int m = CP / 2; m >= 1; m >>= 1)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-          for (int g = 0; g < NT; ++g) s[u][g] += __shfl_xor(s[u][g], m, kWave);
+        for (int g = 0; g < NT; ++g) s[u][g] = group_sum<CP>(s[u][g]);
       const int col = column(blk, 0);
       if (part == 0 && col < col_end) {
 #pragma unroll

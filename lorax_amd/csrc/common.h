@@ -124,43 +124,132 @@ __device__ __forceinline__ typename D::vec8 zero8() {
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
+// Cross-lane sums without the LDS crossbar.  __shfl_xor compiles to ds_bpermute_b32, an LDS instruction with an
+// address register and a round trip through the LDS pipeline; every lane distance the reductions of these kernels
+// use has a cheaper form on gfx950:
+//   1, 2     DPP quad_perm (folds into the add that consumes it)
+//   4        two DPP row shifts, each writing the banks (groups of four lanes) it serves
+//   8        DPP row_ror:8
+//   16, 32   v_permlane16_swap / v_permlane32_swap, which exchange half of one register with half of another:
+//            with (a, b) in, r0 + r1 out is a + a(lane ^ M) in the lanes whose bit M is clear and b + b(lane ^ M)
+//            in the others - the exchange step of a transposing reduction in two instructions, no select.
+// Results are bit-identical to the __shfl_xor forms: the same two values are added (fp32 add commutes).
+template <int CTRL, int BANKS>
+__device__ __forceinline__ float dpp_move(float old, float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v),
+                                                               CTRL, 0xF, BANKS, false));
+}
+// v of lane (lane ^ M), M in {1, 2, 4, 8}.
+template <int M>
+__device__ __forceinline__ float lane_xor_dpp(float v) {
+  static_assert(M == 1 || M == 2 || M == 4 || M == 8, "DPP reaches lanes of the same row of 16");
+  if constexpr (M == 1) return dpp_move<0xB1, 0xF>(v, v);  // quad_perm [1, 0, 3, 2]
+  if constexpr (M == 2) return dpp_move<0x4E, 0xF>(v, v);  // quad_perm [2, 3, 0, 1]
+  if constexpr (M == 8) return dpp_move<0x128, 0xF>(v, v);  // row_ror:8
+  // M == 4: lanes 0-3 and 8-11 of a row take lane + 4 (row_shl:4), lanes 4-7 and 12-15 take lane - 4 (row_shr:4)
+  const float up = dpp_move<0x104, 0x5>(v, v);
+  return dpp_move<0x114, 0xA>(up, v);
+}
+// keep + send(lane ^ M), where a lane keeps lo and sends hi if its bit M is clear, and keeps hi and sends lo if set.
+template <int M>
+__device__ __forceinline__ float fold_pair(float lo, float hi, bool upper) {
+  if constexpr (M == 32) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi),
+                                                    false, false);
+    // (elements copied out before the bit casts: a bit cast applied to r[1] directly reads r[0])
+    const unsigned r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+  } else if constexpr (M == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi),
+                                                    false, false);
+    const unsigned r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+  } else {
+    const float keep = upper ? hi : lo;
+    const float send = upper ? lo : hi;
+    return keep + lane_xor_dpp<M>(send);
+  }
+}
+// v + v(lane ^ M)
+template <int M>
+__device__ __forceinline__ float xor_add(float v) {
+  if constexpr (M >= 16) return fold_pair<M>(v, v, false);
+  else return v + lane_xor_dpp<M>(v);
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave with DPP row shifts and the two row broadcasts (six VALU
+// instructions of a few cycles each where six __shfl_up are six dependent trips through the LDS crossbar).
+template <int CTRL, int ROWS>
+__device__ __forceinline__ int dpp_add_from(int v) {
+  // lanes whose source is outside the row (or whose row is masked off) add nothing
+  return v + __builtin_amdgcn_update_dpp(0, v, CTRL, ROWS, 0xF, true);
+}
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  v = dpp_add_from<0x111, 0xF>(v);  // row_shr:1
+  v = dpp_add_from<0x112, 0xF>(v);  // row_shr:2
+  v = dpp_add_from<0x114, 0xF>(v);  // row_shr:4
+  v = dpp_add_from<0x118, 0xF>(v);  // row_shr:8 - every row of 16 lanes now holds its own prefix sums
+  v = dpp_add_from<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3: + total of the row before
+  v = dpp_add_from<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3: + total of rows 0 and 1
+  return v;
+}
+// v of lane `src`, src wave-uniform.
+__device__ __forceinline__ int read_lane(int v, int src) {
+  return __builtin_amdgcn_readlane(v, __builtin_amdgcn_readfirstlane(src));
+}
+
 // Sum over the 64 lanes of a wave; every lane receives the total.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+  v = xor_add<32>(v);
+  v = xor_add<16>(v);
+  v = xor_add<8>(v);
+  v = xor_add<4>(v);
+  v = xor_add<2>(v);
+  return xor_add<1>(v);
+}
+
+// Sum over aligned groups of CP lanes (CP a power of two <= 16); every lane of a group receives its total.
+// Distances from CP / 2 down to 1, the order the kernels have always added in.
+template <int CP>
+__device__ __forceinline__ float group_sum(float v) {
+  static_assert(CP >= 1 && CP <= 16 && (CP & (CP - 1)) == 0, "CP must be a power of two <= 16");
+  if constexpr (CP >= 16) v = xor_add<8>(v);
+  if constexpr (CP >= 8) v = xor_add<4>(v);
+  if constexpr (CP >= 4) v = xor_add<2>(v);
+  if constexpr (CP >= 2) v = xor_add<1>(v);
   return v;
 }
 
-// Reduces N per-lane values across the wave with N-1+log2(64/N) shuffles instead of
+// Reduces N per-lane values across the wave with N-1+log2(64/N) exchanges instead of
 // 6*N: at every step a lane hands half of its values to the partner lane and keeps
 // the sum of the other half.  On return lane l holds in vals[0] the wave-wide total
 // of the input value with index transpose_reduce_index<N>(l).
+template <int M, int N>
+__device__ __forceinline__ void transpose_reduce_step(float (&vals)[N], int n, bool upper) {
+  const int half = n >> 1;
+#pragma unroll
+  for (int i = 0; i < N / 2; ++i) {
+    if (i < half) {
+      float lo = vals[i];
+      float hi = vals[i + half];
+      // Opaque to the optimiser: without this it rewrites "upper ? vals[i + half] : vals[i]"
+      // into a load with a lane-dependent index, which costs an N-way select chain per access.
+      asm volatile("" : "+v"(lo), "+v"(hi));
+      vals[i] = fold_pair<M>(lo, hi, upper);
+    }
+  }
+}
 template <int N>
 __device__ __forceinline__ void transpose_reduce(float (&vals)[N]) {
   static_assert(N >= 1 && N <= 64 && (N & (N - 1)) == 0, "N must be a power of two <= 64");
   const int lane = lane_id();
-  int n = N;
-  int m = 32;
-#pragma unroll
-  for (; n > 1; n >>= 1, m >>= 1) {
-    const bool upper = (lane & m) != 0;
-    const int half = n >> 1;
-#pragma unroll
-    for (int i = 0; i < N / 2; ++i) {
-      if (i < half) {
-        float lo = vals[i];
-        float hi = vals[i + half];
-        // Opaque to the optimiser: without this it rewrites "upper ? vals[i + half] : vals[i]"
-        // into a load with a lane-dependent index, which costs an N-way select chain per access.
-        asm volatile("" : "+v"(lo), "+v"(hi));
-        const float keep = upper ? hi : lo;
-        const float send = upper ? lo : hi;
-        vals[i] = keep + __shfl_xor(send, m, kWave);
-      }
-    }
-  }
-#pragma unroll
-  for (; m >= 1; m >>= 1) vals[0] += __shfl_xor(vals[0], m, kWave);
+  // distance 32 with n = N values, 16 with N / 2, ...; once one value is left the remaining distances are plain sums
+  if constexpr (N >= 2) transpose_reduce_step<32>(vals, N, (lane & 32) != 0); else vals[0] = xor_add<32>(vals[0]);
+  if constexpr (N >= 4) transpose_reduce_step<16>(vals, N / 2, (lane & 16) != 0); else vals[0] = xor_add<16>(vals[0]);
+  if constexpr (N >= 8) transpose_reduce_step<8>(vals, N / 4, (lane & 8) != 0); else vals[0] = xor_add<8>(vals[0]);
+  if constexpr (N >= 16) transpose_reduce_step<4>(vals, N / 8, (lane & 4) != 0); else vals[0] = xor_add<4>(vals[0]);
+  if constexpr (N >= 32) transpose_reduce_step<2>(vals, N / 16, (lane & 2) != 0); else vals[0] = xor_add<2>(vals[0]);
+  if constexpr (N >= 64) transpose_reduce_step<1>(vals, N / 32, (lane & 1) != 0); else vals[0] = xor_add<1>(vals[0]);
 }
 
 // Index of the input value whose total lane `lane` holds after transpose_reduce<N>.

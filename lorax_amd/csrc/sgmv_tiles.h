@@ -35,28 +35,22 @@ __device__ __forceinline__ int merged_tile_count(int len, int rows_per_tile) {
 template <bool MERGE = false>
 __device__ __forceinline__ bool tile_in_chunk(int s, int e, int seg0, int rows_per_tile, int tile, int& base,
                                               RowTile& out) {
-  const int lane = lane_id();
   const int len = max(e - s, 0);
   const int nt = MERGE ? merged_tile_count(len, rows_per_tile) : (len + rows_per_tile - 1) / rows_per_tile;
-  int inc = nt;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const int t = __shfl_up(inc, d, kWave);
-    if (lane >= d) inc += t;
-  }
-  const int chunk_total = __shfl(inc, kWave - 1, kWave);
+  const int inc = wave_inclusive_scan(nt);
+  const int chunk_total = __builtin_amdgcn_readlane(inc, kWave - 1);
   const int rel = tile - base;
   if (rel < chunk_total) {
     const bool hit = (rel >= inc - nt) && (rel < inc);
     const uint64_t mask = __ballot(hit);
     const int src = __ffsll(static_cast<unsigned long long>(mask)) - 1;
-    const int ti = rel - __shfl(inc - nt, src, kWave);
-    const int s_f = __shfl(s, src, kWave);
-    const int e_f = __shfl(e, src, kWave);
+    const int ti = rel - read_lane(inc - nt, src);
+    const int s_f = read_lane(s, src);
+    const int e_f = read_lane(e, src);
     out.seg = seg0 + src;
     out.index = ti;
     if (MERGE) {
-      const int nt_f = __shfl(nt, src, kWave);
+      const int nt_f = read_lane(nt, src);
       const int blocks = (e_f - s_f + 15) / 16;
       out.row0 = s_f + 16 * static_cast<int>(static_cast<int64_t>(ti) * blocks / nt_f);
       out.row_end = min(e_f, s_f + 16 * static_cast<int>(static_cast<int64_t>(ti + 1) * blocks / nt_f));
