@@ -1,13 +1,14 @@
 """Benchmark of the multi-adapter LoRA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {all,1,2,3,4,5,mid}] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {all,1,2,3,4,5,mid,5dec}] [--layers L]
 
 A step is one pass of one synthetic batch through the LoRA computation of `layers` decoder
 layers (every projection of the configuration), issued through the reference-shaped API and
 replayed as one HIP graph, with all inputs resident in HBM.
 
-With no --config the run measures the five benchmark configurations one after the other (and one
-mid-size prefill batch) and prints ONE JSON line.  Its top level is the BGMV decode configuration
+With no --config the run measures the five benchmark configurations one after the other (and, under
+"extra", one mid-size prefill batch and the decode tokens of configuration 5 on their own as a decode
+batch) and prints ONE JSON line.  Its top level is the BGMV decode configuration
 (cfg2: 256 bf16 tokens over 128 resident rank-8 adapters, 5 % of the tokens without adapter, LoRA
 on q/k/v/o): metric/value = tokens x layers per second of the whole step over exactly K steps.
 "configs" holds the same figures for every configuration; "roofline_min" the lowest HBM-roofline
@@ -42,7 +43,7 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
-    p.add_argument("--config", default="all", choices=["all", "1", "2", "3", "4", "5", "mid"])
+    p.add_argument("--config", default="all", choices=["all", "1", "2", "3", "4", "5", "mid", "5dec"])
     p.add_argument("--windows", type=int, default=5, help="timing windows of --steps steps per configuration")
     p.add_argument("--cpu-budget", type=float, default=0.0,
                    help="seconds of host time for the CPU baseline of one configuration (0 = the default share)")
@@ -60,9 +61,9 @@ def parse_args():
     return p.parse_args()
 
 
-DEFAULT_LAYERS = {"1": 32, "2": 32, "3": 8, "4": 2, "5": 1, "mid": 16}
+DEFAULT_LAYERS = {"1": 32, "2": 32, "3": 8, "4": 2, "5": 1, "mid": 16, "5dec": 1}
 # seconds of host time the CPU baseline of each configuration may take in the default run
-CPU_BUDGET_S = {"1": 2.0, "2": 5.0, "3": 5.0, "4": 6.0, "5": 6.0, "mid": 2.0}
+CPU_BUDGET_S = {"1": 2.0, "2": 5.0, "3": 5.0, "4": 6.0, "5": 6.0, "mid": 2.0, "5dec": 4.0}
 GATED = ("1", "2", "3", "4")  # configurations whose roofline fractions feed roofline_min
 
 
@@ -72,6 +73,8 @@ def build_workload(cfg: str, layers: int, device):
     L = layers or DEFAULT_LAYERS[cfg]
     if cfg == "mid":
         return synthetic.mid_prefill(device, num_layers=L, weights_on_device=True)
+    if cfg == "5dec":
+        return synthetic.config5_decode(device, num_layers=L, weights_on_device=True)
     return synthetic.CONFIGS[int(cfg)](device, num_layers=L, weights_on_device=True)
 
 
@@ -197,37 +200,61 @@ class Plan:
 
     def _add_sgmv_group(self, x, y, h_in, r, jobs):
         """Shrink of up to four projections in one launch (x counted once; it overwrites v, no zero-fill), then
-        one expand per projection from the resident B^T stacks."""
+        one expand per projection from the resident B^T stacks.  Where the tables list many segments of a few
+        rows last and carry a routing plan for them (decode tokens inside a prefill batch), the segment kernels
+        take the long segments and one batched per-token shrink and expand take the rest, as lorax_amd.layers."""
         import torch
 
         from lorax_amd import _native, sgmv
 
         e = 2
         first = jobs[0][0]
-        starts, ends = first.segment_starts, first.segment_ends
+        plans = [rd.short_plan for rd, _, _ in jobs]
+        split = all(p is not None for p in plans)
+        n_long = first.num_long_segments if split else first.segment_starts.numel()
+        starts, ends = first.segment_starts[:n_long], first.segment_ends[:n_long]
         lens = (ends - starts).clamp(min=0)
         rows = int(lens.sum().item())
         flat = torch.zeros((len(jobs), x.size(0), r), dtype=x.dtype, device=x.device)
         vs = list(flat.unbind(0))
-        tables = [rd.lora_a_t_ptr for rd, _, _ in jobs]
+        tables = [rd.lora_a_t_ptr[:n_long] for rd, _, _ in jobs]
         tmp_s = sgmv.get_shrink_scratch(x.device)
         shrink_bytes = shrink_gather = rows * h_in * e
-        for rd, _, _ in jobs:
-            uniq = len(set(rd.lora_a_t_ptr[lens > 0].tolist()))
+        for table in tables:
+            uniq = len(set(table[lens > 0].tolist()))
             shrink_bytes += uniq * r * h_in * e + rows * r * e
             shrink_gather += rows * r * h_in * e + rows * r * e
         self.calls.append(("sgmv_shrink",
                            lambda layer: _native.sgmv_shrink_multi(vs, x, tables, starts, ends, tmp_s, layer, 1.0, False),
                            shrink_bytes, 2 * rows * r * h_in * len(jobs), shrink_gather))
+        if split:
+            # rows and distinct adapters of the plan: record = [count, 4 rows, A address, B address, 0]
+            counts = [(int(p[:, 0].sum().item()), len(set(p[:, 5].tolist()))) for p in plans]
+            n0 = counts[0][0]
+            self.calls.append((
+                "bgmv_shrink",
+                lambda layer: _native.bgmv_multi([(v, x, None, None, 0, None) for v in vs], layer, 1.0, False, plans),
+                n0 * h_in * e + sum(u * r * h_in * e + n * r * e for n, u in counts),
+                sum(2 * n * r * h_in for n, _ in counts),
+                n0 * h_in * e + sum(n * r * h_in * e + n * r * e for n, _ in counts)))
         for v, (rd, off, size) in zip(vs, jobs):
-            uniq = len(set(rd.lora_b_t_ptr[lens > 0].tolist()))
+            b_table = rd.lora_b_t_ptr[:n_long]
+            tmp_e = rd.tmp_expand[: sgmv.get_tmp_expand_size(n_long)]
+            uniq = len(set(b_table[lens > 0].tolist()))
 
-            def expand(layer, v=v, rd=rd, off=off, size=size):
-                sgmv.lora_b_sgmv_cutlass_slice(y, v, rd.tmp_expand, rd.lora_b_t_ptr, rd.segment_starts,
-                                               rd.segment_ends, layer, off, size, transposed=True)
+            def expand(layer, v=v, b_table=b_table, tmp_e=tmp_e, off=off, size=size):
+                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_table, starts, ends, layer, off, size, transposed=True)
 
             self.calls.append(("sgmv_expand", expand, rows * r * e + uniq * r * size * e + 2 * rows * size * e,
                                2 * rows * r * size, rows * r * e + rows * r * size * e + 2 * rows * size * e))
+        if split:
+            problems = [(y, v, None, None, off, size) for v, (_, off, size) in zip(vs, jobs)]
+            sizes = [size for _, _, size in jobs]
+            self.calls.append((
+                "bgmv_expand", lambda layer: _native.bgmv_multi(problems, layer, 1.0, True, plans),
+                sum(n * r * e + u * r * size * e + 2 * n * size * e for (n, u), size in zip(counts, sizes)),
+                sum(2 * n * r * size for (n, _), size in zip(counts, sizes)),
+                sum(n * r * e + n * r * size * e + 2 * n * size * e for (n, _), size in zip(counts, sizes))))
 
     def _add_sgmv_fused(self, x, y, h_in, r, jobs):
         """Shrink and expand of up to four projections of a short prefill batch in one launch; v stays on chip."""
@@ -555,7 +582,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    todo = ["2", "1", "3", "4", "5", "mid"] if args.config == "all" else [args.config]
+    todo = ["2", "1", "3", "4", "5", "mid", "5dec"] if args.config == "all" else [args.config]
     records = {}
     for cfg in todo:
         print(f"bench: configuration {cfg}", file=sys.stderr, flush=True)
@@ -585,8 +612,8 @@ def main():
         "cpu_baseline": head["cpu_baseline"],
     }
     if args.config == "all":
-        out["configs"] = {f"cfg{k}": records[k] for k in todo if k != "mid"}
-        out["extra"] = {"mid_prefill_1k": records["mid"]}
+        out["configs"] = {f"cfg{k}": records[k] for k in todo if k not in ("mid", "5dec")}
+        out["extra"] = {"mid_prefill_1k": records["mid"], "cfg5_decode_tokens_bgmv": records["5dec"]}
         fracs = [(f"cfg{k}", kind, rec["frac"], records[k]["roofline"]["bound"])
                  for k in GATED for kind, rec in records[k]["kernels"].items()]
         lowest = min(fracs, key=lambda t: t[2])

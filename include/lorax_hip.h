@@ -294,14 +294,16 @@ typedef struct lorax_table_group {
   int32_t rank;
   int32_t use_sgmv;     /* 1: segment tables (prefill, or a rank above 128); 0: per-token */
   int32_t num_segments; /* entries of the group's pointer tables                          */
-  int32_t num_chunks;   /* routing-plan records (use_sgmv = 0)                            */
-  int32_t reserved;
+  int32_t num_chunks;   /* routing-plan records: of all routed tokens (use_sgmv = 0), of the rows of
+                           the group's short segments (use_sgmv = 1, 0 = no such plan)            */
+  int32_t num_long_segments; /* use_sgmv = 1 with a plan: the tables list the segments of more than 4
+                           rows first, this many; the plan covers the rest.  Else num_segments    */
   int64_t a_ptr_off;    /* int64[num_segments] stack addresses per segment                */
   int64_t b_ptr_off;
   int64_t starts_off;   /* int32[num_segments] (use_sgmv = 1), else -1                    */
   int64_t ends_off;
   int64_t indices_off;  /* int64[num_tokens] slot in the group's tables or -1 (use_sgmv = 0) */
-  int64_t plan_off;     /* int64[num_chunks][8] routing plan (use_sgmv = 0)               */
+  int64_t plan_off;     /* int64[num_chunks][8] routing plan, -1 = none                   */
 } lorax_table_group_t;
 
 int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t num_tokens,

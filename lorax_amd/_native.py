@@ -66,7 +66,7 @@ class TableGroup(ctypes.Structure):
     """lorax_table_group_t of include/lorax_hip.h."""
 
     _fields_ = [("layer_type", _c.c_int32), ("rank", _c.c_int32), ("use_sgmv", _c.c_int32),
-                ("num_segments", _c.c_int32), ("num_chunks", _c.c_int32), ("reserved", _c.c_int32),
+                ("num_segments", _c.c_int32), ("num_chunks", _c.c_int32), ("num_long_segments", _c.c_int32),
                 ("a_ptr_off", _c.c_int64), ("b_ptr_off", _c.c_int64), ("starts_off", _c.c_int64),
                 ("ends_off", _c.c_int64), ("indices_off", _c.c_int64), ("plan_off", _c.c_int64)]
 
@@ -266,7 +266,8 @@ def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> N
     that share the token count and the direction; shrink problems share x.shape and may differ in rank
     (y's width), expand problems may differ in rank (x's width) and output width.  y_slice_size None means
     the whole width of y.
-    `plans`, if given, holds one routing plan per problem: an int64 device tensor [num_groups, 8]."""
+    `plans`, if given, holds one routing plan per problem: an int64 device tensor [num_groups, 8]; w_ptr and
+    indicies of a planned problem may then be None (the kernels read the plan only)."""
     if not 1 <= len(problems) <= MAX_BGMV_PROBLEMS:
         raise RuntimeError(f"between 1 and {MAX_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
     arr = (BgmvProblem * len(problems))()
@@ -274,17 +275,21 @@ def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> N
     for i, (y, x, w_ptr, indicies, y_offset, y_slice_size) in enumerate(problems):
         _check_input(y, "y", 2)
         _check_input(x, "x", 2)
-        _check_input(w_ptr, "w_ptr", 1)
-        _check_input(indicies, "indicies", 1)
-        _check_same(y, x, w_ptr, indicies)
-        if w_ptr.dtype != torch.int64 or indicies.dtype != torch.int64:
-            raise RuntimeError("w_ptr and indicies must be int64 tensors")
+        planned_only = plans is not None and w_ptr is None and indicies is None  # the plan holds the routing
+        if planned_only:
+            _check_same(y, x)
+        else:
+            _check_input(w_ptr, "w_ptr", 1)
+            _check_input(indicies, "indicies", 1)
+            _check_same(y, x, w_ptr, indicies)
+            if w_ptr.dtype != torch.int64 or indicies.dtype != torch.int64:
+                raise RuntimeError("w_ptr and indicies must be int64 tensors")
         if x.size(0) != x0.size(0) or x.dtype != x0.dtype or x.device != x0.device:
             raise RuntimeError("all problems of one launch must have inputs of one row count, dtype and device")
-        if indicies.size(0) != x.size(0) or y.size(0) != x.size(0):
+        if (not planned_only and indicies.size(0) != x.size(0)) or y.size(0) != x.size(0):
             raise RuntimeError(
                 f"CHECK_EQ(indicies.size(0), x.size(0)) / CHECK_EQ(y.size(0), x.size(0)) failed. "
-                f"{indicies.size(0)}, {y.size(0)} vs {x.size(0)}"
+                f"{'-' if planned_only else indicies.size(0)}, {y.size(0)} vs {x.size(0)}"
             )
         h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
         plan_ptr, num_groups = None, 0
@@ -296,7 +301,8 @@ def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> N
             plan_ptr, num_groups = plan.data_ptr(), plan.size(0)
             if num_groups == 0:
                 plan_ptr = x.data_ptr()  # an empty plan has no storage; any non-null address will do
-        arr[i] = BgmvProblem(y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), indicies.data_ptr(), int(y_offset),
+        arr[i] = BgmvProblem(y.data_ptr(), x.data_ptr(), None if planned_only else w_ptr.data_ptr(),
+                             None if planned_only else indicies.data_ptr(), int(y_offset),
                              y.size(1), h_out, plan_ptr, num_groups, x.size(1))
     with torch.cuda.device(x0.device):
         rc = lib().lorax_bgmv_multi(arr, len(problems), x0.size(0), x0.size(1), int(layer_idx), float(scale),

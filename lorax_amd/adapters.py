@@ -191,7 +191,8 @@ class RankSegments:
                  tmp_expand: Optional[torch.Tensor], segment_starts: Optional[torch.Tensor],
                  segment_ends: Optional[torch.Tensor], indices: Optional[torch.Tensor],
                  plan: Optional[torch.Tensor] = None, lora_a_t_ptr: Optional[torch.Tensor] = None,
-                 lora_b_t_ptr: Optional[torch.Tensor] = None, segments_key=None):
+                 lora_b_t_ptr: Optional[torch.Tensor] = None, segments_key=None,
+                 num_long_segments: Optional[int] = None, short_plan: Optional[torch.Tensor] = None):
         self.rank = rank
         self._lora_a_ptr = lora_a_ptr  # a tensor, or a function that builds it
         self._lora_b_ptr = lora_b_ptr
@@ -213,6 +214,12 @@ class RankSegments:
         # prefill: hashable and equal for rank groups (of different layer types) whose segment_starts /
         # segment_ends hold the same values - their shrinks can share one pass over x; None = unknown
         self.segments_key = segments_key
+        # prefill: a batch with many segments of a few rows (decode tokens inside a prefill batch) lists them
+        # last in its tables and, besides, as a routing plan over their rows (records as in `plan`).  A caller
+        # may then run the segment kernels over the first num_long_segments entries only and the per-token
+        # kernels over short_plan; the tables as a whole stay complete.  None / the table's length: no such plan.
+        self.short_plan = short_plan
+        self.num_long_segments = num_long_segments
 
     @property
     def lora_a_ptr(self) -> Optional[torch.Tensor]:
@@ -248,6 +255,30 @@ def build_bgmv_plan(token_slots: List[int], a_addrs: List[int], b_addrs: List[in
     return records
 
 
+SHORT_SEGMENT_ROWS = 4    # segments of at most this many rows may go to the per-token kernels ...
+MIN_SHORT_SEGMENTS = 32   # ... when a rank group has at least this many of them
+
+
+def build_short_plan(segs: List[int], bounds: List[int], a_addrs: List[int], b_addrs: List[int],
+                     owners: List[int]) -> List[List[int]]:
+    """Plan records over the rows of the segments `segs` (each of at most SHORT_SEGMENT_ROWS rows; the segments
+    of one owner next to each other): the rows of one owner, in the order given, in chunks of BGMV_PLAN_GROUP.
+    a_addrs / b_addrs / owners are indexed by segment."""
+    records = []
+    i = 0
+    while i < len(segs):
+        j, rows = i, []
+        while j < len(segs) and owners[segs[j]] == owners[segs[i]]:
+            rows += list(range(bounds[segs[j]], bounds[segs[j] + 1]))
+            j += 1
+        for k in range(0, len(rows), BGMV_PLAN_GROUP):
+            chunk = rows[k : k + BGMV_PLAN_GROUP]
+            pad = [chunk[0]] * (BGMV_PLAN_GROUP - len(chunk))
+            records.append([len(chunk), *chunk, *pad, a_addrs[segs[i]], b_addrs[segs[i]], 0])
+        i = j
+    return records
+
+
 def pad_bgmv_plan(plan: torch.Tensor, num_records: int) -> torch.Tensor:
     """`plan` extended with all-zero records to a fixed number of records: the kernels skip them, so a decode
     step captured in a graph can be replayed with the plans of later batches copied into the same tensor
@@ -259,13 +290,18 @@ def pad_bgmv_plan(plan: torch.Tensor, num_records: int) -> torch.Tensor:
     return padded
 
 
-def _segment_order(segs: List[int], seg_adapters: List[int], bounds: List[int]):
+def _count_short(segs: List[int], bounds: List[int]) -> int:
+    return sum(1 for s in segs if bounds[s + 1] - bounds[s] <= SHORT_SEGMENT_ROWS)
+
+
+def _segment_order(segs: List[int], seg_adapters: List[int], bounds: List[int], split: bool = False):
     """Sort key of a rank group's segments: rows of the segment's adapter inside the group, descending, then the
-    adapter index."""
+    adapter index; with `split`, the segments of more than SHORT_SEGMENT_ROWS rows before the others."""
     rows: Dict[int, int] = defaultdict(int)
     for s in segs:
         rows[seg_adapters[s]] += bounds[s + 1] - bounds[s]
-    return lambda s: (-rows[seg_adapters[s]], seg_adapters[s])
+    return lambda s: (split and bounds[s + 1] - bounds[s] <= SHORT_SEGMENT_ROWS, -rows[seg_adapters[s]],
+                      seg_adapters[s])
 
 
 class _LayoutView(Mapping):
@@ -399,11 +435,20 @@ class BatchLoraWeights(BatchAdapterWeights):
                     group_a[s], group_b[s] = a_c.data_ptr(), b_c.data_ptr()
             group_a_ptr = lora_a_t_ptr if chunk is None else torch.tensor(group_a, dtype=torch.int64, device=device)
             group_b_ptr = lora_b_t_ptr if chunk is None else torch.tensor(group_b, dtype=torch.int64, device=device)
+            num_long = short_plan = None
             if use_sgmv:
                 # the order of a group's segments is free: keep the segments of one adapter together, so that
                 # their tiles run back to back and share the adapter's weights in L2, adapters with the most
-                # rows first (the long tiles of a launch start early)
-                segs.sort(key=_segment_order(segs, seg_adapters, meta.adapter_segments.tolist()))
+                # rows first (the long tiles of a launch start early); many segments of a few rows go last and
+                # get a routing plan for the per-token kernels
+                seg_bounds = meta.adapter_segments.tolist()
+                n_short = _count_short(segs, seg_bounds) if head_starts is None else 0
+                split = n_short >= MIN_SHORT_SEGMENTS
+                segs.sort(key=_segment_order(segs, seg_adapters, seg_bounds, split))
+                if split:
+                    num_long = len(segs) - n_short
+                    records = build_short_plan(segs[num_long:], seg_bounds, group_a, group_b, seg_adapters)
+                    short_plan = torch.tensor(records, dtype=torch.int64, device=device).reshape(-1, BGMV_PLAN_WORDS)
             tmp_shrink = tmp_expand = starts = ends = token_slots = plan = None
             if use_sgmv:
                 tmp_shrink, tmp_expand = get_tmp_tensors(len(segs), rank, device)
@@ -444,6 +489,8 @@ class BatchLoraWeights(BatchAdapterWeights):
                 lora_a_t_ptr=group_a_ptr[segs] if use_sgmv else None,
                 lora_b_t_ptr=group_b_ptr[segs] if use_sgmv else None,
                 segments_key=(tuple(segs), head_starts is not None, chunk) if use_sgmv else None,
+                num_long_segments=num_long if num_long is not None else (len(segs) if use_sgmv else None),
+                short_plan=short_plan,
             )
 
         return cls(
@@ -682,7 +729,9 @@ def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAda
                     # the group's segments in the builder's order (only computed if somebody asks for the
                     # reference-layout tables)
                     segs = [s for s, a in enumerate(seg_adapters) if a in loras and loras[a].lora_a_r == rank]
-                    segs.sort(key=_segment_order(segs, seg_adapters, bounds.tolist()))
+                    seg_bounds = bounds.tolist()
+                    split = _count_short(segs, seg_bounds) >= MIN_SHORT_SEGMENTS
+                    segs.sort(key=_segment_order(segs, seg_adapters, seg_bounds, split))
                     return table(layout)[segs]
 
                 rank_data[g.rank] = RankSegments(
@@ -698,6 +747,9 @@ def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAda
                     lora_b_t_ptr=b_ptr,
                     segments_key=(packed[g.starts_off : g.starts_off + 4 * n].tobytes(),
                                   packed[g.ends_off : g.ends_off + 4 * n].tobytes()),
+                    num_long_segments=g.num_long_segments,
+                    short_plan=dev64[g.plan_off // 8 : g.plan_off // 8 + g.num_chunks * BGMV_PLAN_WORDS].view(
+                        g.num_chunks, BGMV_PLAN_WORDS) if g.plan_off >= 0 else None,
                 )
             else:
                 rank_data[g.rank] = RankSegments(

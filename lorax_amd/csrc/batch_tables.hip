@@ -16,6 +16,12 @@ namespace {
 
 constexpr int kPlanGroup = 4;   // tokens per routing-plan record
 constexpr int kBgmvMaxRank = 128;  // BGMV_MAX_RANK, lorax_server/utils/punica.py:39
+// Decode tokens inside a prefill batch are segments of one row (a speculating request: a few).  The segment
+// kernels give every such segment a row tile of its own; the per-token kernels stream an adapter's weights at a
+// higher rate and once for up to kPlanGroup rows.  A rank group with at least kMinShortSegments segments of at
+// most kShortSegmentRows rows therefore gets them listed last in its tables and, besides, as a routing plan.
+constexpr int kShortSegmentRows = 4;
+constexpr int kMinShortSegments = 32;
 
 struct Packer {
   char* base;
@@ -118,13 +124,22 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
       // weights in L2 - decode tokens inside a prefill batch are one-row segments, and an adapter that serves
       // several of them would otherwise be streamed once per token.  Adapters with the most rows come first,
       // so that the long tiles of a launch start early.  Stable: (rows of the adapter, descending; adapter).
+      int32_t n_short = 0;
+      bool split = false;
       if (use_sgmv) {
         // rows per adapter, indexed by the adapter's position in this layer type's entry list
         entry_rows.assign(count, 0);
         for (int32_t x : segs) entry_rows[seg_entry[x] - type_first] += segment_bounds[x + 1] - segment_bounds[x];
         std::vector<int64_t> rows_of(num_segments, 0);
         for (int32_t x : segs) rows_of[x] = entry_rows[seg_entry[x] - type_first];
+        for (int32_t x : segs) n_short += segment_bounds[x + 1] - segment_bounds[x] <= kShortSegmentRows;
+        split = n_short >= kMinShortSegments;
         std::stable_sort(segs.begin(), segs.end(), [&](int32_t x, int32_t y) {
+          if (split) {  // long segments first, short ones after them
+            const bool sx = segment_bounds[x + 1] - segment_bounds[x] <= kShortSegmentRows;
+            const bool sy = segment_bounds[y + 1] - segment_bounds[y] <= kShortSegmentRows;
+            if (sx != sy) return sy;
+          }
           if (rows_of[x] != rows_of[y]) return rows_of[x] > rows_of[y];
           return segment_owners[x] < segment_owners[y];
         });
@@ -144,6 +159,7 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
         }
       }
       desc.starts_off = desc.ends_off = desc.indices_off = desc.plan_off = -1;
+      desc.num_long_segments = n;
       if (use_sgmv) {
         desc.starts_off = pack.reserve(static_cast<int64_t>(n) * 4);
         desc.ends_off = pack.reserve(static_cast<int64_t>(n) * 4);
@@ -152,6 +168,45 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
           for (int32_t i = 0; i < n; ++i) {
             st[i] = segment_bounds[segs[i]];
             en[i] = segment_bounds[segs[i] + 1];
+          }
+        }
+        if (split) {
+          // Routing plan of the short segments' rows: the segments of one adapter are neighbours in the table
+          // (the sort above), in token order; their rows are cut into records of up to kPlanGroup.
+          const int32_t n_long = n - n_short;
+          desc.num_long_segments = n_long;
+          int32_t chunks = 0;
+          for (int32_t i = n_long; i < n;) {
+            int32_t rows = 0, j = i;
+            for (; j < n && seg_entry[segs[j]] == seg_entry[segs[i]]; ++j)
+              rows += segment_bounds[segs[j] + 1] - segment_bounds[segs[j]];
+            chunks += (rows + kPlanGroup - 1) / kPlanGroup;
+            i = j;
+          }
+          desc.num_chunks = chunks;
+          desc.plan_off = pack.reserve(static_cast<int64_t>(chunks) * lorax::kPlanRecordWords * 8);
+          if (int64_t* rec = pack.at<int64_t>(desc.plan_off)) {
+            for (int32_t i = n_long; i < n;) {
+              const lorax_adapter_entry_t* e = seg_entry[segs[i]];
+              int cnt = 0;
+              auto flush = [&]() {
+                rec[0] = cnt;
+                for (int q = cnt; q < kPlanGroup; ++q) rec[1 + q] = rec[1];
+                rec[5] = e->a_addr;
+                rec[6] = e->b_addr;
+                rec[7] = 0;
+                rec += lorax::kPlanRecordWords;
+                cnt = 0;
+              };
+              int32_t j = i;
+              for (; j < n && seg_entry[segs[j]] == e; ++j)
+                for (int32_t t = segment_bounds[segs[j]]; t < segment_bounds[segs[j] + 1]; ++t) {
+                  rec[1 + cnt++] = t;
+                  if (cnt == kPlanGroup) flush();
+                }
+              if (cnt > 0) flush();
+              i = j;
+            }
           }
         }
       } else {

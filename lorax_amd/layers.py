@@ -35,6 +35,7 @@ from lorax_amd._native import MAX_SGMV_SHRINK_PROBLEMS
 from lorax_amd.sgmv import (
     MAX_RANK_CUSTOM,
     get_shrink_scratch,
+    get_tmp_expand_size,
     has_sgmv,
     lora_a_sgmv_cutlass,
     lora_a_sgmv_resident,
@@ -171,14 +172,30 @@ class LoraLinear(nn.Module):
             for i in range(0, len(group), step):
                 chunk = group[i : i + step]
                 first = chunk[0][0]
+                # Many segments of a few rows (decode tokens inside a prefill batch): the tables list them last and
+                # a routing plan covers their rows.  The segment kernels then take the long segments only and the
+                # per-token kernels the rest - they stream an adapter's weights faster than one row tile per
+                # segment can, and once for up to four rows.  Both write disjoint rows of v and of the result.
+                plans = [rs.short_plan for rs, _, _ in chunk]
+                split = all(p is not None for p in plans)
+                n_long = first.num_long_segments if split else first.segment_starts.numel()
+                starts, ends = first.segment_starts[:n_long], first.segment_ends[:n_long]
                 vs = lora_a_sgmv_resident_multi(
-                    input, get_shrink_scratch(input.device), [rs.lora_a_t_ptr for rs, _, _ in chunk],
-                    first.segment_starts, first.segment_ends, self.layer_id, r, zero_fill=False,
+                    input, get_shrink_scratch(input.device), [rs.lora_a_t_ptr[:n_long] for rs, _, _ in chunk],
+                    starts, ends, self.layer_id, r, zero_fill=False,
                 )
+                if split:
+                    _native.bgmv_multi([(v, input, None, None, 0, None) for v in vs], self.layer_id, 1.0,
+                                       accumulate=False, plans=plans)
                 for v, (rs, start, width) in zip(vs, chunk):
                     lora_b_sgmv_cutlass_slice(
-                        result, v, rs.tmp_expand, rs.lora_b_t_ptr, rs.segment_starts, rs.segment_ends,
+                        result, v, rs.tmp_expand[: get_tmp_expand_size(n_long)], rs.lora_b_t_ptr[:n_long], starts, ends,
                         self.layer_id, start, width, transposed=True,
+                    )
+                if split:
+                    _native.bgmv_multi(
+                        [(result, v, None, None, start, width) for v, (_, start, width) in zip(vs, chunk)],
+                        self.layer_id, 1.0, accumulate=True, plans=plans,
                     )
 
         if stacked_jobs:  # the reference calls add_lora once per projection (utils/layers.py:92-104)

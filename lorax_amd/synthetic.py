@@ -76,11 +76,13 @@ class Workload:
 
 def _splice_rank_group(rs, layer, rank: int, extra) -> None:
     """Adds the segments `extra` to one rank group's tables: the first one in front of the group's second
-    segment, the others at the end."""
+    segment, the others at the end - of the long segments, when the group lists its short segments last and
+    routes them through a plan (the segment kernels then see the added entries too)."""
     from lorax_amd.sgmv import get_tmp_tensors
 
     n = rs.segment_starts.numel()
-    at = [min(1, n)] + [n] * (len(extra) - 1)  # insertion points in the original table
+    n_long = rs.num_long_segments if rs.short_plan is not None else n
+    at = [min(1, n_long)] + [n_long] * (len(extra) - 1)  # insertion points in the original table
 
     def spliced(table, values, dtype):
         parts, prev = [], 0
@@ -107,6 +109,7 @@ def _splice_rank_group(rs, layer, rank: int, extra) -> None:
     rs.segment_starts = spliced(rs.segment_starts, [s for s, _, _ in extra], torch.int32)
     rs.segment_ends = spliced(rs.segment_ends, [e for _, e, _ in extra], torch.int32)
     rs.tmp_shrink, rs.tmp_expand = get_tmp_tensors(n + len(extra), rank, rs.segment_starts.device)
+    rs.num_long_segments = n_long + len(extra)
     if rs.segments_key is not None:
         rs.segments_key = (rs.segments_key, tuple(extra))
 
@@ -265,6 +268,24 @@ def config5(device, num_layers: int = 1, weights_on_device: bool = True, prefill
     w = Workload("cfg5_llama70b_mixed_prefill_decode", torch.bfloat16, torch.device(device), num_layers, True,
                  groups if groups is not None else LLAMA70B_LAYER, idx, rank_of)
     w.extra_segments = [(prefill_tokens // 2, prefill_tokens // 2, dec[0]), (-1, -1, None)]
+    _populate(w, 1005, weights_on_device)
+    return w
+
+
+def config5_decode(device, num_layers: int = 1, weights_on_device: bool = True, decode_tokens: int = 256,
+                   num_adapters: int = 256, groups: Optional[List[ProjectionGroup]] = None,
+                   resident_only_active: bool = False) -> Workload:
+    """The decode tokens of the mixed Llama-70B batch on their own, as a decode batch (per-token routing, BGMV):
+    the same adapter draw as config5, `num_adapters` resident rank-128 adapters, four tokens without adapter."""
+    gen = torch.Generator(device="cpu").manual_seed(1005)
+    dec = torch.randint(0, num_adapters, (decode_tokens,), generator=gen).tolist()
+    idx = dec[: decode_tokens // 2] + [-1] * 4 + dec[decode_tokens // 2 :]
+    rank_of = {a: 128 for a in range(num_adapters)}
+    if resident_only_active:
+        active = set(idx)
+        rank_of = {a: r for a, r in rank_of.items() if a in active}
+    w = Workload("cfg5_llama70b_decode_tokens_bgmv", torch.bfloat16, torch.device(device), num_layers, False,
+                 groups if groups is not None else LLAMA70B_LAYER, idx, rank_of)
     _populate(w, 1005, weights_on_device)
     return w
 

@@ -151,6 +151,37 @@ def test_config5_mlp_projections_reduced():
     _check_workload(w, 0, 0.25)
 
 
+def test_config5_many_decode_tokens_take_the_per_token_kernels():
+    # enough one-row segments for the tables to list them last with a routing plan: the segment kernels then run
+    # the long segments (the added empty ones among them) and the per-token kernels the decode rows
+    groups = [g for g in synthetic.LLAMA70B_LAYER if g.name in ("qkv", "down_proj")]
+    w = synthetic.config5(DEV, num_layers=1, weights_on_device=False, prefill_tokens=200, decode_tokens=44,
+                          num_adapters=12, groups=groups)
+    batch = w.batch_data()
+    for name in ("q_proj", "down_proj"):
+        rd = batch.data[name][LORA].rank_data[128]
+        lens = (rd.segment_ends - rd.segment_starts).tolist()
+        assert rd.short_plan is not None and 0 < rd.num_long_segments < len(lens)
+        assert all(n > 4 or n <= 0 for n in lens[: rd.num_long_segments])  # long runs and the two empty entries
+        assert all(1 <= n <= 4 for n in lens[rd.num_long_segments :])
+        assert int(rd.short_plan[:, 0].sum()) == sum(lens[rd.num_long_segments :])
+    assert_has_empty_segments(w, batch)
+    _check_workload(w, 0, 0.25)
+
+
+def test_config5_decode_tokens_alone_as_bgmv_reduced():
+    # the decode share of the mixed batch as a decode batch: rank 128, the real hidden sizes, fewer tokens
+    for names in (("qkv", "o_proj"), ("gate_up", "down_proj")):
+        groups = [g for g in synthetic.LLAMA70B_LAYER if g.name in names]
+        w = synthetic.config5_decode(DEV, num_layers=1, weights_on_device=False, decode_tokens=20, num_adapters=8,
+                                     groups=groups)
+        batch = w.batch_data()
+        data = batch.data[groups[0].layer_names[0]][LORA]
+        assert not data.use_sgmv and list(data.rank_data) == [128]
+        assert (data.rank_data[128].indices < 0).sum().item() == 4
+        _check_workload(w, 0, 0.25)
+
+
 @pytest.mark.parametrize("prefill", [True, False])
 def test_lm_head_with_a_large_vocabulary(prefill):
     """The LM head through MultiAdapterHead: 70 000 output columns (more than the reference's BGMV kernels take),

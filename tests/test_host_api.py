@@ -349,7 +349,7 @@ def test_prefill_tables_touch_only_resident_layouts():
     assert torch.equal(lws[0].weights_a.transpose(1, 2), lws[0].weights_a_t)
 
 
-@pytest.mark.parametrize("config", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("config", [1, 2, 3, 4, 5, "5 with many decode tokens"])
 def test_native_table_builder_matches_python_tables(config):
     """lorax_build_batch_tables (one call, one packed buffer for all layer types) against the per-layer-type Python
     restatement of BatchLoraWeights.load, which the golden vectors of the reference's test_lora.py pin."""
@@ -364,6 +364,10 @@ def test_native_table_builder_matches_python_tables(config):
         kwargs.update(num_tokens=96, num_adapters=40)
     if config == 5:
         kwargs.update(prefill_tokens=50, decode_tokens=24, num_adapters=12)
+    many_short = config == "5 with many decode tokens"
+    if many_short:  # enough one-row segments for the tables to list them last and to carry a plan for them
+        config = 5
+        kwargs.update(prefill_tokens=50, decode_tokens=70, num_adapters=12)
     w = synthetic.CONFIGS[config]("cpu", **kwargs)
     fast = AdapterBatchData.from_meta(w.meta, w.weights, prefill=w.prefill)
     assert set(fast.data) == {n for n, lw in w.weights.items() if not lw.is_empty()}
@@ -378,7 +382,10 @@ def test_native_table_builder_matches_python_tables(config):
         assert a.adapter_index_configs.keys() == b.adapter_index_configs.keys()
         for rank in a.rank_data:
             ra, rb = a.rank_data[rank], b.rank_data[rank]
-            for field in ("lora_a_t_ptr", "lora_b_t_ptr", "segment_starts", "segment_ends", "indices", "plan"):
+            assert ra.num_long_segments == rb.num_long_segments
+            assert (ra.short_plan is not None) == many_short
+            for field in ("lora_a_t_ptr", "lora_b_t_ptr", "segment_starts", "segment_ends", "indices", "plan",
+                          "short_plan"):
                 ta, tb = getattr(ra, field), getattr(rb, field)
                 assert (ta is None) == (tb is None), field
                 if ta is not None:
@@ -386,6 +393,54 @@ def test_native_table_builder_matches_python_tables(config):
             assert torch.equal(ra.lora_a_ptr, rb.lora_a_ptr) and torch.equal(ra.lora_b_ptr, rb.lora_b_ptr)
     bounds, owners = find_segments(w.meta.adapter_indices)
     assert w.meta.adapter_segments.tolist() == bounds and w.meta.segment_indices == owners
+
+
+def test_short_segments_of_a_prefill_batch_get_a_plan():
+    """A prefill batch with at least 32 segments of at most 4 rows lists them after the long segments and carries
+    a routing plan over exactly their rows: every such row once, under its own adapter's stack addresses, at most
+    four rows per record, the rows of one adapter together; the tables as a whole still hold every segment."""
+    from lorax_amd.adapters import BatchLoraWeights, LayerAdapterWeights, LoraConfig, LoraWeights
+    from lorax_amd.synthetic import make_meta
+
+    h, L, r = 32, 1, 16
+    layer = LayerAdapterWeights()
+    for idx in range(6):
+        layer.add_adapter(idx, LoraWeights([torch.randn(h, r)] * L, [torch.randn(r, h)] * L, LoraConfig(r=r)))
+    gen = torch.Generator().manual_seed(5)
+    idx = [0] * 40 + [1] * 7  # two long runs
+    for _ in range(40):       # then runs of 1 to 4 rows
+        a = int(torch.randint(0, 6, (1,), generator=gen))
+        idx += [a] * int(torch.randint(1, 5, (1,), generator=gen))
+        idx += [-1]           # separated by a row without adapter, so that equal neighbours do not merge
+    meta = make_meta(idx, torch.device("cpu"))
+    rd = BatchLoraWeights.load(layer.adapter_weights, meta, "q_proj", True, None).rank_data[r]
+    starts, ends = rd.segment_starts.tolist(), rd.segment_ends.tolist()
+    lens = [e - s for s, e in zip(starts, ends)]
+    n_long = rd.num_long_segments
+    assert 0 < n_long < len(lens) and rd.short_plan is not None
+    assert all(n > 4 for n in lens[:n_long]) and all(1 <= n <= 4 for n in lens[n_long:])
+    routed = sorted(t for s, e in zip(starts, ends) for t in range(s, e))
+    assert routed == [t for t, a in enumerate(idx) if a >= 0]  # the tables as a whole are complete
+    short_rows = sorted(t for s, e in zip(starts[n_long:], ends[n_long:]) for t in range(s, e))
+    plan = rd.short_plan.tolist()
+    seen, owners_in_order = [], []
+    for n, t0, t1, t2, t3, a_addr, b_addr, zero in plan:
+        assert 1 <= n <= 4 and zero == 0
+        rows = [t0, t1, t2, t3][:n]
+        assert [t0, t1, t2, t3][n:] == [t0] * (4 - n)  # unused slots repeat the first row
+        owner = {idx[t] for t in rows}
+        assert len(owner) == 1
+        lw = layer.adapter_weights[owner.pop()]
+        assert (a_addr, b_addr) == (lw.weights_a_t.data_ptr(), lw.weights_b_t.data_ptr())
+        seen += rows
+        owners_in_order.append(idx[rows[0]])
+    assert sorted(seen) == short_rows and len(seen) == len(set(seen))
+    runs = [a for i, a in enumerate(owners_in_order) if i == 0 or owners_in_order[i - 1] != a]
+    assert len(runs) == len(set(runs))  # the records of one adapter are neighbours
+    # fewer short segments than the threshold: no plan, every segment "long"
+    meta = make_meta([0] * 9 + [1, -1, 2, 2, -1, 3], torch.device("cpu"))
+    rd = BatchLoraWeights.load(layer.adapter_weights, meta, "q_proj", True, None).rank_data[r]
+    assert rd.short_plan is None and rd.num_long_segments == rd.segment_starts.numel() == 4
 
 
 def test_native_table_builder_reports_the_space_it_needs():
