@@ -135,8 +135,7 @@ class Plan:
                         self._add_sgmv_fused(x, y, group.h_in, r, same[i:i + _native.MAX_FUSED_BGMV_PROBLEMS])
                     continue
                 step = max(1, min(_native.MAX_SGMV_SHRINK_PROBLEMS, 128 // r))
-                for i in range(0, len(same), step):
-                    self._add_sgmv_group(x, y, group.h_in, r, same[i:i + step])
+                self._add_sgmv_group(x, y, group.h_in, r, same, step)
             all_jobs = [(r, rd, off, size) for r, rank_jobs in decode.items() for rd, off, size in rank_jobs]
             all_fused = bool(all_jobs) and self.use_plan and self.fuse_small_ranks and all(
                 _native.bgmv_lora_fits(r, group.h_in, size) for r, _, _, size in all_jobs)
@@ -198,11 +197,12 @@ class Plan:
         self.calls.append(("sgmv_expand", expand, rows * r * e + uniq * r * size * e + 2 * rows * size * e,
                            2 * rows * r * size, rows * r * e + rows * r * size * e + 2 * rows * size * e))
 
-    def _add_sgmv_group(self, x, y, h_in, r, jobs):
-        """Shrink of up to four projections in one launch (x counted once; it overwrites v, no zero-fill), then
-        one expand per projection from the resident B^T stacks.  Where the tables list many segments of a few
-        rows last and carry a routing plan for them (decode tokens inside a prefill batch), the segment kernels
-        take the long segments and one batched per-token shrink and expand take the rest, as lorax_amd.layers."""
+    def _add_sgmv_group(self, x, y, h_in, r, jobs, step):
+        """Projections of one rank with the same segment tables, as lorax_amd.layers runs them: shrinks of `step`
+        projections per launch (x counted once per launch; they overwrite v, no zero-fill), then one expand per
+        projection from the resident B^T stacks.  Where the tables list many segments of a few rows last and carry
+        a routing plan for them (decode tokens inside a prefill batch), the segment kernels take the long segments
+        and ONE batched per-token shrink and ONE batched per-token expand take the rest, for all projections."""
         import torch
 
         from lorax_amd import _native, sgmv
@@ -217,16 +217,19 @@ class Plan:
         rows = int(lens.sum().item())
         flat = torch.zeros((len(jobs), x.size(0), r), dtype=x.dtype, device=x.device)
         vs = list(flat.unbind(0))
-        tables = [rd.lora_a_t_ptr[:n_long] for rd, _, _ in jobs]
         tmp_s = sgmv.get_shrink_scratch(x.device)
-        shrink_bytes = shrink_gather = rows * h_in * e
-        for table in tables:
-            uniq = len(set(table[lens > 0].tolist()))
-            shrink_bytes += uniq * r * h_in * e + rows * r * e
-            shrink_gather += rows * r * h_in * e + rows * r * e
-        self.calls.append(("sgmv_shrink",
-                           lambda layer: _native.sgmv_shrink_multi(vs, x, tables, starts, ends, tmp_s, layer, 1.0, False),
-                           shrink_bytes, 2 * rows * r * h_in * len(jobs), shrink_gather))
+        for i in range(0, len(jobs), step):
+            tables = [rd.lora_a_t_ptr[:n_long] for rd, _, _ in jobs[i:i + step]]
+            shrink_bytes = shrink_gather = rows * h_in * e
+            for table in tables:
+                uniq = len(set(table[lens > 0].tolist()))
+                shrink_bytes += uniq * r * h_in * e + rows * r * e
+                shrink_gather += rows * r * h_in * e + rows * r * e
+
+            def shrink(layer, out=vs[i:i + step], tables=tables):
+                _native.sgmv_shrink_multi(out, x, tables, starts, ends, tmp_s, layer, 1.0, False)
+
+            self.calls.append(("sgmv_shrink", shrink, shrink_bytes, 2 * rows * r * h_in * len(tables), shrink_gather))
         if split:
             # rows and distinct adapters of the plan: record = [count, 4 rows, A address, B address, 0]
             counts = [(int(p[:, 0].sum().item()), len(set(p[:, 5].tolist()))) for p in plans]

@@ -39,7 +39,6 @@ from lorax_amd.sgmv import (
     has_sgmv,
     lora_a_sgmv_cutlass,
     lora_a_sgmv_resident,
-    lora_a_sgmv_resident_multi,
     lora_b_sgmv_cutlass,
     lora_b_sgmv_cutlass_slice,
     resident_shrink_applies,
@@ -168,34 +167,40 @@ class LoraLinear(nn.Module):
                         input, first.segment_starts, first.segment_ends, r, self.layer_id,
                     )
                 continue
+            # Many segments of a few rows (decode tokens inside a prefill batch): the tables list them last and a
+            # routing plan covers their rows.  The segment kernels then take the long segments only and the
+            # per-token kernels the rest - they stream an adapter's weights faster than one row tile per segment
+            # can, and once for up to four rows.  Both write disjoint rows of v and of the result.
+            first = group[0][0]
+            plans = [rs.short_plan for rs, _, _ in group]
+            split = all(p is not None for p in plans)
+            n_long = first.num_long_segments if split else first.segment_starts.numel()
+            starts, ends = first.segment_starts[:n_long], first.segment_ends[:n_long]
+            # v needs no zero-fill: the shrinks overwrite the rows of their segments and the expands read no others
+            flat = torch.empty((len(group), input.size(0), r), dtype=input.dtype, device=input.device)
+            vs = list(flat.unbind(0))
             step = max(1, min(MAX_SGMV_SHRINK_PROBLEMS, MAX_RANK_CUSTOM // r))
             for i in range(0, len(group), step):
-                chunk = group[i : i + step]
-                first = chunk[0][0]
-                # Many segments of a few rows (decode tokens inside a prefill batch): the tables list them last and
-                # a routing plan covers their rows.  The segment kernels then take the long segments only and the
-                # per-token kernels the rest - they stream an adapter's weights faster than one row tile per
-                # segment can, and once for up to four rows.  Both write disjoint rows of v and of the result.
-                plans = [rs.short_plan for rs, _, _ in chunk]
-                split = all(p is not None for p in plans)
-                n_long = first.num_long_segments if split else first.segment_starts.numel()
-                starts, ends = first.segment_starts[:n_long], first.segment_ends[:n_long]
-                vs = lora_a_sgmv_resident_multi(
-                    input, get_shrink_scratch(input.device), [rs.lora_a_t_ptr[:n_long] for rs, _, _ in chunk],
-                    starts, ends, self.layer_id, r, zero_fill=False,
+                _native.sgmv_shrink_multi(
+                    vs[i : i + step], input, [rs.lora_a_t_ptr[:n_long] for rs, _, _ in group[i : i + step]],
+                    starts, ends, get_shrink_scratch(input.device), self.layer_id, 1.0, False,
                 )
-                if split:
-                    _native.bgmv_multi([(v, input, None, None, 0, None) for v in vs], self.layer_id, 1.0,
-                                       accumulate=False, plans=plans)
-                for v, (rs, start, width) in zip(vs, chunk):
-                    lora_b_sgmv_cutlass_slice(
-                        result, v, rs.tmp_expand[: get_tmp_expand_size(n_long)], rs.lora_b_t_ptr[:n_long], starts, ends,
-                        self.layer_id, start, width, transposed=True,
-                    )
-                if split:
+            batch = _native.MAX_BGMV_PROBLEMS
+            if split:  # the short rows of every projection of the group in one launch
+                for i in range(0, len(group), batch):
+                    _native.bgmv_multi([(v, input, None, None, 0, None) for v in vs[i : i + batch]], self.layer_id,
+                                       1.0, accumulate=False, plans=plans[i : i + batch])
+            for v, (rs, start, width) in zip(vs, group):
+                lora_b_sgmv_cutlass_slice(
+                    result, v, rs.tmp_expand[: get_tmp_expand_size(n_long)], rs.lora_b_t_ptr[:n_long], starts, ends,
+                    self.layer_id, start, width, transposed=True,
+                )
+            if split:
+                for i in range(0, len(group), batch):
                     _native.bgmv_multi(
-                        [(result, v, None, None, start, width) for v, (_, start, width) in zip(vs, chunk)],
-                        self.layer_id, 1.0, accumulate=True, plans=plans,
+                        [(result, v, None, None, start, width)
+                         for v, (_, start, width) in zip(vs[i : i + batch], group[i : i + batch])],
+                        self.layer_id, 1.0, accumulate=True, plans=plans[i : i + batch],
                     )
 
         if stacked_jobs:  # the reference calls add_lora once per projection (utils/layers.py:92-104)
