@@ -320,13 +320,17 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_
   constexpr int R = NB * 16;
   int kparts = 1;
   const int nst_all = a.d_in / kLdsKc;
-  if (a.partials != nullptr && (tiles <= 128 || tuning().shrink_ksplit > 0)) {
-    kparts = static_cast<int>(256 / tiles);
+  // Up to 128 tiles: about one workgroup per CU.  Up to 192 tiles (a single long run of a few thousand rows cut
+  // into 32-row tiles): two or three parts, about two workgroups per CU - measured on a 4096-row run at rank 128,
+  // 140 tiles: 51 -> 40 us over h_in = 8192 and 145 -> 86 us over h_in = 28672 with three parts (two: 45 and 116 us;
+  // four and more, which no longer fit the CUs at once: 46 and 104 us).  Launches with more tiles than that are
+  // slower with parts than without (254 tiles in two parts: 27 against 23 us).
+  if (a.partials != nullptr && (tiles < 192 || tuning().shrink_ksplit > 0)) {
+    kparts = static_cast<int>((tiles <= 128 ? 256 : 512) / tiles);
     if (kparts > 8) kparts = 8;
     if (kparts > nst_all / 8) kparts = nst_all / 8;
     if (tuning().shrink_ksplit > 0) kparts = tuning().shrink_ksplit < nst_all ? tuning().shrink_ksplit : nst_all;
-    const size_t room = a.partial_bytes < kPartialBytes ? a.partial_bytes : kPartialBytes;
-    while (kparts > 1 && static_cast<size_t>(kparts) * a.num_tokens * R * sizeof(float) > room) --kparts;
+    while (kparts > 1 && static_cast<size_t>(kparts) * a.num_tokens * R * sizeof(float) > a.partial_bytes) --kparts;
     if (kparts < 1) kparts = 1;
   }
   const int64_t wgs = tiles * kparts;
