@@ -280,6 +280,13 @@ size_t lorax_sgmv_tmp_size(int32_t num_problems);
  *   used); `groups`: one descriptor per (layer type, rank), ranks in order of first appearance, with byte
  *   offsets into `packed`.  Returns LORAX_ESPACE when `packed` or `groups` is too small (or NULL), with
  *   *packed_bytes and *num_groups set to what is needed.
+ * Segment tables (use_sgmv = 1) keep the segments of one adapter next to each other (the order of a group's
+ *   segments is free).  A group with at least 32 segments of at most 4 rows - decode tokens inside a prefill
+ *   batch - lists those after the longer ones and also gets a routing plan over their rows (records as for
+ *   lorax_bgmv_multi): a caller may run lorax_sgmv_shrink / lorax_sgmv_expand over the first
+ *   num_long_segments entries and lorax_bgmv_multi over the plan, on the same v and y, instead of the segment
+ *   kernels over the whole table.  The reference routes every row of such a batch through its segment kernels
+ *   (lorax_server/adapters/lora.py:279, server/lorax_server/models/flash_causal_lm.py:1594).
  */
 typedef struct lorax_adapter_entry {
   int64_t adapter; /* adapter index as it appears in adapter_indices            */
