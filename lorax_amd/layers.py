@@ -180,7 +180,8 @@ class LoraLinear(nn.Module):
             flat = torch.empty((len(group), input.size(0), r), dtype=input.dtype, device=input.device)
             vs = list(flat.unbind(0))
             step = max(1, min(MAX_SGMV_SHRINK_PROBLEMS, MAX_RANK_CUSTOM // r))
-            for i in range(0, len(group), step):
+            # (no long segment at all: the per-token launches do the whole update)
+            for i in range(0, len(group) if n_long > 0 else 0, step):
                 _native.sgmv_shrink_multi(
                     vs[i : i + step], input, [rs.lora_a_t_ptr[:n_long] for rs, _, _ in group[i : i + step]],
                     starts, ends, get_shrink_scratch(input.device), self.layer_id, 1.0, False,
@@ -190,7 +191,7 @@ class LoraLinear(nn.Module):
                 for i in range(0, len(group), batch):
                     _native.bgmv_multi([(v, input, None, None, 0, None) for v in vs[i : i + batch]], self.layer_id,
                                        1.0, accumulate=False, plans=plans[i : i + batch])
-            for v, (rs, start, width) in zip(vs, group):
+            for v, (rs, start, width) in zip(vs, group) if n_long > 0 else ():
                 lora_b_sgmv_cutlass_slice(
                     result, v, rs.tmp_expand[: get_tmp_expand_size(n_long)], rs.lora_b_t_ptr[:n_long], starts, ends,
                     self.layer_id, start, width, transposed=True,

@@ -169,6 +169,25 @@ def test_config5_many_decode_tokens_take_the_per_token_kernels():
     _check_workload(w, 0, 0.25)
 
 
+def test_prefill_batch_of_short_segments_only():
+    """A prefill batch whose segments all have one to four rows (many requests with tiny prompts): the tables hold
+    no long segment at all and the per-token kernels do the whole update."""
+    gen = torch.Generator().manual_seed(21)
+    idx = []
+    for _ in range(40):
+        a = int(torch.randint(0, 6, (1,), generator=gen))
+        idx += [a] * int(torch.randint(1, 5, (1,), generator=gen)) + [-1]
+    groups = [synthetic.ProjectionGroup("qkv", ["q_proj", "k_proj", "v_proj"], 1024, [1024, 256, 256]),
+              synthetic.ProjectionGroup("o_proj", ["o_proj"], 1024, [1024])]
+    w = synthetic.Workload("short_segments_only", torch.bfloat16, torch.device(DEV), 1, True, groups, idx,
+                           {a: 32 for a in range(6)})
+    synthetic._populate(w, 21, False)
+    batch = w.batch_data()
+    rd = batch.data["q_proj"][LORA].rank_data[32]
+    assert rd.short_plan is not None and rd.num_long_segments == 0
+    _check_workload(w, 0, 0.25)
+
+
 def test_config5_decode_tokens_alone_as_bgmv_reduced():
     # the decode share of the mixed batch as a decode batch: rank 128, the real hidden sizes, fewer tokens
     for names in (("qkv", "o_proj"), ("gate_up", "down_proj")):
