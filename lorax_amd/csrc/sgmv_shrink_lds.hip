@@ -306,10 +306,15 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_
     rows_per_tile = (tuning().shrink_rows + 15) / 16 * 16;
   }
   // Tiles of 48 rows in buffers of 48: the fourth row block of 64-row buffers would be staged (re-reading the
-  // tile's last row) and multiplied for nothing.
-  if constexpr (MBLK == 4 && (KSPLIT || NB % 4 == 0)) {
-    if (rows_per_tile == 48 && fixed_rows == 0 && tuning().shrink_mb == 0)
-      return launch_lds_m<D, NB, 3, KSPLIT>(a, stream, 48);
+  // tile's last row) and multiplied for nothing.  With three row blocks the waves take k slices at every rank
+  // (96 accumulator registers per lane at rank 128; cfg3's stacked gate/up launch 37.0 -> 34.8 us against the
+  // waves splitting the output blocks).
+  if constexpr (MBLK == 4) {
+    constexpr bool kSlices = KSPLIT || NB > 4;
+    if constexpr (kSlices || NB % 4 == 0) {  // (output blocks of three row blocks only divide as 1 x 4)
+      if (rows_per_tile == 48 && fixed_rows == 0 && tuning().shrink_mb == 0)
+        return launch_lds_m<D, NB, 3, kSlices>(a, stream, 48);
+    }
   }
   const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
   // K parts: a workgroup streams its tile's x and A at about 50 GB/s whatever the launch, so a launch of a
