@@ -255,6 +255,22 @@ def test_ranks_above_the_kernel_limit_run_as_rank_chunks(mode, lens):
     """Adapters of rank 192 and 256 next to one of rank 16 and requests without adapter, on a fused q/k/v
     projection: the kernels take ranks up to 128, so such an adapter is served as chunks of its rank (128 + 64,
     128 + 128), each a rank group of its own.  The oracle multiplies with the whole rank at once."""
+    _check_rank_chunks(mode, [0, 1, 2, 9, 1, 0, 2, 2, 9, 0, 1, 1], lens)      # 9 has no weights
+
+
+def test_rank_chunks_with_many_short_segments():
+    """The same in a prefill batch with dozens of one- to three-row segments per chunked adapter: every chunk's
+    rank group lists them last and routes them through the per-token kernels, chunk after chunk."""
+    adapters, lens = [0, 1], [60, 20]
+    for i in range(40):
+        adapters += [0, 9, 1, 9]
+        lens += [1 + i % 3, 1, 1 + (i + 1) % 3, 2]
+    batch = _check_rank_chunks("prefill", adapters, lens)
+    for key, rs in batch.data["q_proj"][LORA].rank_data.items():
+        assert (rs.short_plan is not None) == isinstance(key, tuple), key  # adapter 2 (rank 16) is not in the batch
+
+
+def _check_rank_chunks(mode, request_adapters, lens):
     from lorax_amd.adapters import AdapterBatchData, LayerAdapterWeights, LoraConfig, LoraWeights
     from lorax_amd.synthetic import make_meta
 
@@ -262,7 +278,6 @@ def test_ranks_above_the_kernel_limit_run_as_rank_chunks(mode, lens):
     dtype, hidden, layers, layer_id = torch.bfloat16, 1024, 2, 1
     names, sizes = ["q_proj", "k_proj", "v_proj"], [1024, 256, 256]
     gen = torch.Generator().manual_seed(len(lens) + sum(lens))
-    request_adapters = [0, 1, 2, 9, 1, 0, 2, 2, 9, 0, 1, 1]      # 9 has no weights
     ranks = {0: 192, 1: 256, 2: 16}
     tokens = [a for a, n in zip(request_adapters, lens) for _ in range(n)]
     meta = make_meta(tokens, torch.device(DEV))
@@ -276,8 +291,9 @@ def test_ranks_above_the_kernel_limit_run_as_rank_chunks(mode, lens):
         weights[name] = layer
     batch = AdapterBatchData.from_meta(meta, weights, prefill=prefill)
     groups = batch.data["q_proj"][LORA].rank_data
-    assert sorted(map(str, groups)) == sorted(map(str, [16, (192, 0), (192, 1), (256, 0), (256, 1)]))
-    assert sorted(rs.rank for rs in groups.values()) == [16, 64, 128, 128, 128]
+    expect = [(192, 0), (192, 1), (256, 0), (256, 1)] + ([16] if 2 in request_adapters else [])
+    assert sorted(map(str, groups)) == sorted(map(str, expect))
+    assert sorted(rs.rank for rs in groups.values()) == ([16] if 2 in request_adapters else []) + [64, 128, 128, 128]
     assert batch.data["q_proj"][LORA].use_sgmv == prefill
 
     T = len(tokens)
@@ -297,3 +313,4 @@ def test_ranks_above_the_kernel_limit_run_as_rank_chunks(mode, lens):
     assert_close(out, ref, f"rank chunks, {mode}", rounded=[delta, delta])
     untouched = torch.tensor([a not in ranks for a in tokens])
     assert torch.equal(out.cpu()[untouched], y0[untouched])
+    return batch
