@@ -94,9 +94,9 @@ int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* ind
  * expand problems may differ in rank (the problem's own h_in field) and in h_out - so the rank
  * groups of a multi-rank batch (lorax_server/adapters/lora.py:339-348, one kernel call per rank
  * in the reference) go out in ONE shrink launch and ONE expand launch.  Each problem is computed
- * exactly as by lorax_bgmv.  accumulate = 0 (shrink launches only) stores
- * dtype(sum) instead of adding it, so the caller need not zero v first; rows of tokens whose
- * index is negative are not written in either mode.
+ * exactly as by lorax_bgmv.  accumulate = 0 stores dtype(sum) instead of adding it (meant for
+ * shrink launches, so that the caller need not zero v first; an expand launch takes it too); rows
+ * of tokens whose index is negative are not written in either mode.
  *
  * Routing plan (optional).  Finding which tokens share an adapter costs every workgroup a scan
  * of indices[]; a caller that builds the index tables on the host anyway (as the reference does,

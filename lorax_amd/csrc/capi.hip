@@ -159,8 +159,6 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
   if (!planned) a.grid_rows = num_tokens;
   a.work_rows = planned ? a.grid_rows : (num_tokens + 1) / 2;
   if (a.grid_rows == 0) return LORAX_OK;
-  if (!a.expand && accumulate != 0 && accumulate != 1)
-    return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (accumulate != 0 && accumulate != 1)
     return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (num_tokens > 65535)

@@ -57,7 +57,7 @@ struct BgmvArgs {
   int64_t work_rows;  // estimate of the rows that have work (sizes the rows-per-workgroup choice)
   int64_t layer_idx;
   float scale;
-  int accumulate;     // shrink only: 0 = overwrite y, 1 = add to y
+  int accumulate;     // 0 = overwrite the routed rows of y, 1 = add to y
   int dtype;
 };
 

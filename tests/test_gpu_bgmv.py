@@ -168,6 +168,27 @@ def test_bgmv_expand_vector_and_scalar_y_paths_agree_bit_for_bit(dtype, r):
     assert torch.equal(ya.cpu()[idx < 0], y0.cpu()[idx < 0])
 
 
+@pytest.mark.parametrize("r", [8, 64])
+def test_bgmv_expand_overwrite_mode(r):
+    """accumulate = 0 on an expand launch stores the update instead of adding it: the routed rows equal the
+    update added to zeros, the other rows keep what they held."""
+    dtype, T, h_out, n = torch.bfloat16, 37, 1160, 5
+    gen = torch.Generator().manual_seed(700 + r)
+    wb_t = _stacks(n, 1, h_out, r, gen, dtype)
+    v = randn((T, r), 1.0, gen, dtype, DEV)
+    idx = _indices(T, n, gen, drop=0.25)
+    ptrs, idx_d = ptr_table(wb_t, DEV), idx.to(DEV)
+    added = torch.zeros((T, h_out), dtype=dtype, device=DEV)
+    _native.bgmv_multi([(added, v, ptrs, idx_d, 0, None)], 0, 1.0, accumulate=True)
+    junk = randn((T, h_out), 3.0, gen, dtype, DEV)
+    stored = junk.clone()
+    _native.bgmv_multi([(stored, v, ptrs, idx_d, 0, None)], 0, 1.0, accumulate=False)
+    torch.cuda.synchronize()
+    routed = (idx >= 0).to(DEV)
+    assert torch.equal(stored[routed], added[routed]) and torch.count_nonzero(added[routed]) > 0
+    assert torch.equal(stored[~routed], junk[~routed])
+
+
 def test_bgmv_under_graph_capture_replays_identically():
     dtype, T, h_in, h_out, r, n = torch.bfloat16, 64, 4096, 4096, 32, 9
     gen = torch.Generator().manual_seed(3)
