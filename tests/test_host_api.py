@@ -443,6 +443,32 @@ def test_short_segments_of_a_prefill_batch_get_a_plan():
     assert rd.short_plan is None and rd.num_long_segments == rd.segment_starts.numel() == 4
 
 
+@pytest.mark.parametrize("short_segments,rows,expect_plan", [(31, 4, False), (32, 4, True), (40, 5, False), (32, 1, True)])
+def test_short_segment_thresholds_agree_between_the_two_builders(short_segments, rows, expect_plan):
+    """The native builder and its Python restatement keep their own copies of the two thresholds (at least 32
+    segments of at most 4 rows): both sides of both boundaries, compared field by field."""
+    from lorax_amd.adapters import BatchLoraWeights, LayerAdapterWeights, LoraConfig, LoraWeights
+    from lorax_amd.synthetic import make_meta
+
+    h, r = 32, 8
+    layer = LayerAdapterWeights()
+    for idx in range(3):
+        layer.add_adapter(idx, LoraWeights([torch.randn(h, r)], [torch.randn(r, h)], LoraConfig(r=r)))
+    idx = [0] * 20
+    for i in range(short_segments):
+        idx += [1 + i % 2] * rows + [-1]
+    meta = make_meta(idx, torch.device("cpu"))
+    slow = BatchLoraWeights.load(layer.adapter_weights, meta, "q_proj", True, None).rank_data[r]
+    fast = AdapterBatchData.from_meta(meta, {"q_proj": layer}, prefill=True).data["q_proj"][LORA].rank_data[r]
+    assert (slow.short_plan is not None) == expect_plan
+    assert slow.num_long_segments == fast.num_long_segments == (1 if expect_plan else short_segments + 1)
+    for field in ("segment_starts", "segment_ends", "lora_a_t_ptr", "lora_b_t_ptr", "short_plan"):
+        a, b = getattr(slow, field), getattr(fast, field)
+        assert (a is None) == (b is None), field
+        if a is not None:
+            assert torch.equal(a, b), field
+
+
 def test_native_table_builder_reports_the_space_it_needs():
     import ctypes
 
