@@ -335,7 +335,9 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_
     if (kparts > 8) kparts = 8;
     if (kparts > nst_all / 8) kparts = nst_all / 8;
     if (tuning().shrink_ksplit > 0) kparts = tuning().shrink_ksplit < nst_all ? tuning().shrink_ksplit : nst_all;
-    while (kparts > 1 && static_cast<size_t>(kparts) * a.num_tokens * R * sizeof(float) > a.partial_bytes) --kparts;
+    // (the first 8 MiB whatever the buffer's size, so that the result does not depend on it)
+    const size_t room = a.partial_bytes < kPartialBytes ? a.partial_bytes : kPartialBytes;
+    while (kparts > 1 && static_cast<size_t>(kparts) * a.num_tokens * R * sizeof(float) > room) --kparts;
     if (kparts < 1) kparts = 1;
   }
   const int64_t wgs = tiles * kparts;
