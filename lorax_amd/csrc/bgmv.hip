@@ -123,13 +123,71 @@ __device__ __forceinline__ BatchSlot batch_slot(const BgmvBatch& batch, int coun
     const int subs = batch.run_subs[0];
     return BatchSlot{0, v / subs, v % subs};
   }
-  int p = 0;
-  while (p + 1 < count && v >= batch.run_end[p]) ++p;  // first problem of the run that holds v
-  const int rem = v - batch.base[p];
-  const int run_subs = batch.run_subs[p];
+  // Lane i looks at problem i: the five table entries of all problems arrive in one trip to the kernel arguments
+  // (a walk with the scalar unit asks for them one after the other, each answer deciding the next question - a
+  // handful of dependent cache misses in front of the first useful load of every CU's first workgroup).
+  const int i = lane_id() < kMaxBgmvProblems ? lane_id() : kMaxBgmvProblems - 1;
+  const int run_end = batch.run_end[i], base = batch.base[i], subs = batch.run_subs[i];
+  const int sub_lo = batch.sub_lo[i], sub_hi = batch.sub_hi[i];
+  const bool mine = lane_id() < kMaxBgmvProblems && i + 1 < count;
+  // first problem of the run that holds v: run_end does not decrease with the problem number
+  const int first = __popcll(__ballot(mine && v >= run_end));
+  const int rem = v - read_lane(base, first);
+  const int run_subs = read_lane(subs, first);
   const int chunk = rem / run_subs, s = rem % run_subs;
-  while (p + 1 < count && s >= batch.sub_hi[p]) ++p;
-  return BatchSlot{p, chunk, s - batch.sub_lo[p]};
+  // inside the run, sub_hi increases and the run's last problem has sub_hi = run_subs > s
+  const int run_stop = read_lane(run_end, first);
+  const int p = first + __popcll(__ballot(mine && i >= first && run_end == run_stop && s >= sub_hi));
+  return BatchSlot{p, chunk, s - read_lane(sub_lo, p)};
+}
+
+// Problem `p` of a batch, fetched the same way: lane i asks for the fields of problem i before anybody knows p,
+// and the fields of the problem the workgroup turns out to serve are read from that lane.  Indexing the kernel
+// arguments with p instead is one more dependent trip to memory in front of the routing record.  Wave-uniform.
+// Used by the single-launch kernels, whose workgroups are alone on their CU (9.8 -> 9.2 us per decode launch);
+// in the shrink and expand kernels the seventeen registers it holds cost a wave per SIMD and more than it saves
+// (expand 27.0 -> 28.3 us on the mixed-rank decode batch), so they index the arguments.
+__device__ __forceinline__ int64_t read_lane64(int64_t v, int src) {
+  const uint32_t lo = static_cast<uint32_t>(read_lane(static_cast<int>(static_cast<uint32_t>(v)), src));
+  const uint32_t hi = static_cast<uint32_t>(read_lane(static_cast<int>(static_cast<uint64_t>(v) >> 32), src));
+  return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+struct ProblemFields {  // one lane's copy of problem min(lane, 15)
+  int64_t y, x, w_ptrs, indices, y_offset, y_stride, plan;
+  int width, narrow, num_groups;
+};
+__device__ __forceinline__ ProblemFields preload_problems(const BgmvBatch& batch) {
+  const BgmvProblem& q = batch.p[lane_id() < kMaxBgmvProblems ? lane_id() : kMaxBgmvProblems - 1];
+  return ProblemFields{reinterpret_cast<int64_t>(q.y), reinterpret_cast<int64_t>(q.x),
+                       reinterpret_cast<int64_t>(q.w_ptrs), reinterpret_cast<int64_t>(q.indices), q.y_offset,
+                       q.y_stride, reinterpret_cast<int64_t>(q.plan), q.width, q.narrow, q.num_groups};
+}
+__device__ __forceinline__ BgmvProblem select_problem(const ProblemFields& f, int p) {
+  BgmvProblem P;
+  P.y = reinterpret_cast<void*>(read_lane64(f.y, p));
+  P.x = reinterpret_cast<const void*>(read_lane64(f.x, p));
+  P.w_ptrs = reinterpret_cast<const int64_t*>(read_lane64(f.w_ptrs, p));
+  P.indices = reinterpret_cast<const int64_t*>(read_lane64(f.indices, p));
+  P.y_offset = read_lane64(f.y_offset, p);
+  P.y_stride = read_lane64(f.y_stride, p);
+  P.width = read_lane(f.width, p);
+  P.narrow = read_lane(f.narrow, p);
+  P.plan = reinterpret_cast<const int64_t*>(read_lane64(f.plan, p));
+  P.num_groups = read_lane(f.num_groups, p);
+  return P;
+}
+
+// The two fields of a problem that stand between batch_slot and the routing record, fetched like batch_slot's
+// tables (lane i: problem i) and with them: the record's address is then known one trip to memory after the
+// workgroup starts, and the record travels together with the problem's other fields, which the scalar unit reads
+// from the kernel arguments once the problem's number is known.
+struct PlanOfLane {
+  int64_t plan;
+  int num_groups;
+};
+__device__ __forceinline__ PlanOfLane preload_plans(const BgmvBatch& batch) {
+  const BgmvProblem& q = batch.p[lane_id() < kMaxBgmvProblems ? lane_id() : kMaxBgmvProblems - 1];
+  return PlanOfLane{reinterpret_cast<int64_t>(q.plan), q.num_groups};
 }
 
 // Resolves the token chunk of workgroup row `row` and the address of its adapter's stack.
@@ -137,11 +195,13 @@ __device__ __forceinline__ BatchSlot batch_slot(const BgmvBatch& batch, int coun
 // record: [ntok, tok0..tok3, address of the A stack, address of the B^T stack, reserved];
 // without one, the chunk is found by scanning indices[] (group_tokens).  Returns the number of
 // tokens, 0 if the workgroup has nothing to do.  Wave-uniform.
-__device__ __forceinline__ int resolve_chunk(const BgmvProblem& P, int num_tokens, bool expand, int row,
-                                             int (&toks)[kGroup], int64_t& stack_addr) {
-  if (P.plan != nullptr) {
-    if (row >= P.num_groups) return 0;
-    const int64_t* rec = P.plan + static_cast<int64_t>(row) * kPlanRecordWords;
+// `plan` / `num_groups` are the problem's fields of that name, handed over separately because the callers have
+// them before the rest of the problem (PlanOfLane).
+__device__ __forceinline__ int resolve_chunk(const BgmvProblem& P, const int64_t* plan, int num_groups, int num_tokens,
+                                             bool expand, int row, int (&toks)[kGroup], int64_t& stack_addr) {
+  if (plan != nullptr) {
+    if (row >= num_groups) return 0;
+    const int64_t* rec = plan + static_cast<int64_t>(row) * kPlanRecordWords;
     const int n = static_cast<int>(rec[0]);
 #pragma unroll
     for (int g = 0; g < kGroup; ++g) toks[g] = static_cast<int>(rec[1 + g]);
@@ -161,13 +221,16 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_shrink_kernel(
     int accumulate_into_y) {
   __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<RS * kGroup>::value];
   using E = typename D::E;
+  const PlanOfLane plans = preload_plans(batch);
   const BatchSlot slot = batch_slot(batch, count);
   const BgmvProblem& P = batch.p[slot.problem];
   const int r = P.narrow;
   const int row0 = slot.sub * RS;
   int toks[kGroup];
   int64_t stack_addr;
-  const int n = resolve_chunk(P, num_tokens, false, slot.chunk, toks, stack_addr);
+  const int n = resolve_chunk(P, reinterpret_cast<const int64_t*>(read_lane64(plans.plan, slot.problem)),
+                              read_lane(plans.num_groups, slot.problem), num_tokens, false, slot.chunk, toks,
+                              stack_addr);
   if (n == 0) return;
   const E* A = reinterpret_cast<const E*>(stack_addr) + (layer_idx * r + row0) * static_cast<int64_t>(h_in);
   E* Y = static_cast<E*>(P.y);
@@ -435,16 +498,13 @@ __device__ __forceinline__ void bgmv_expand_tokens(typename D::E* Y, const typen
 }
 
 template <typename D, int CP, int U, bool VY>
-__device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const BatchSlot& slot, int num_tokens,
+__device__ __forceinline__ void bgmv_expand_problem(const BgmvProblem& P, const BatchSlot& slot, int n,
+                                                    const int (&toks)[kGroup], int64_t stack_addr,
                                                     int64_t layer_idx, float scale, bool acc_y, float* wave_sums) {
   using E = typename D::E;
   const int h_out = P.width;
   const int r = P.narrow;
   const int col0 = slot.sub * (kBgmvThreads / CP) * U;  // U = expand_steps(CP, the launch's U)
-  int toks[kGroup];
-  int64_t stack_addr;
-  const int n = resolve_chunk(P, num_tokens, true, slot.chunk, toks, stack_addr);
-  if (n == 0) return;
   const E* B = reinterpret_cast<const E*>(stack_addr) + layer_idx * h_out * static_cast<int64_t>(r);
   E* Y = static_cast<E*>(P.y);
   const E* V = static_cast<const E*>(P.x);
@@ -489,23 +549,30 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_expand_kernel(const BgmvBat
   __shared__ __attribute__((aligned(16))) float sums[VY ? (kBgmvThreads / kWave) * kWaveSums : 4];
   float* wave_sums = sums + (VY ? (threadIdx.x / kWave) * kWaveSums : 0);
   const bool acc_y = accumulate_into_y != 0;
+  const PlanOfLane plans = preload_plans(batch);
   const BatchSlot vb = batch_slot(batch, count);
   const BgmvProblem& P = batch.p[vb.problem];
+  // the routing record is asked for before the problem's rank is looked at: it travels with the problem's fields
+  int toks[kGroup];
+  int64_t stack;
+  const int n = resolve_chunk(P, reinterpret_cast<const int64_t*>(read_lane64(plans.plan, vb.problem)),
+                              read_lane(plans.num_groups, vb.problem), num_tokens, true, vb.chunk, toks, stack);
+  if (n == 0) return;
   switch (expand_lanes_per_column(P.narrow)) {
     case 1:
-      bgmv_expand_problem<D, 1, U, VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
+      bgmv_expand_problem<D, 1, U, VY>(P, vb, n, toks, stack, layer_idx, scale, acc_y, wave_sums);
       break;
     case 2:
-      bgmv_expand_problem<D, 2, U, VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
+      bgmv_expand_problem<D, 2, U, VY>(P, vb, n, toks, stack, layer_idx, scale, acc_y, wave_sums);
       break;
     case 4:
-      bgmv_expand_problem<D, 4, expand_steps(4, U), VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
+      bgmv_expand_problem<D, 4, expand_steps(4, U), VY>(P, vb, n, toks, stack, layer_idx, scale, acc_y, wave_sums);
       break;
     case 8:
-      bgmv_expand_problem<D, 8, expand_steps(8, U), VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
+      bgmv_expand_problem<D, 8, expand_steps(8, U), VY>(P, vb, n, toks, stack, layer_idx, scale, acc_y, wave_sums);
       break;
     default:
-      bgmv_expand_problem<D, 16, expand_steps(16, U), VY>(P, vb, num_tokens, layer_idx, scale, acc_y, wave_sums);
+      bgmv_expand_problem<D, 16, expand_steps(16, U), VY>(P, vb, n, toks, stack, layer_idx, scale, acc_y, wave_sums);
       break;
   }
 }
@@ -775,13 +842,14 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch
   using E = typename D::E;
   __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<R * kGroup>::value];
   __shared__ __attribute__((aligned(16))) E vsh[R * kGroup];
+  const ProblemFields fields = preload_problems(batch);  // before anything waits: see select_problem
   VirtualBlock vb;
   if (balanced_chunks > 0) {
     if (!balanced_slot(count, balanced_chunks, chunks_per_xcd, vb)) return;
   } else {
     vb = xcd_virtual_block();
   }
-  const BgmvProblem& P = batch.p[vb.z];
+  const BgmvProblem P = select_problem(fields, vb.z);
   const int h_out = P.width;
   constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
   const int col0 = vb.x * cols_per_wg;
@@ -822,7 +890,15 @@ __global__ __launch_bounds__(kBgmvThreads) void sgmv_lora_rows_kernel(
   __shared__ float red[(kBgmvThreads / kWave) * Pow2Ceil<R * kGroup>::value];
   __shared__ __attribute__((aligned(16))) E vsh[R * kGroup];
   const VirtualBlock vb = xcd_virtual_block();  // x: column slice, y: row chunk, z: projection
-  const SgmvLoraProblem& P = batch.p[vb.z];
+  // lane i fetches problem i's fields, the workgroup's own are read from lane z (see select_problem)
+  const SgmvLoraProblem& mine = batch.p[lane_id() < kMaxSgmvLoraProblems ? lane_id() : kMaxSgmvLoraProblems - 1];
+  SgmvLoraProblem P;
+  P.y = reinterpret_cast<void*>(read_lane64(reinterpret_cast<int64_t>(mine.y), vb.z));
+  P.a_ptrs = reinterpret_cast<const int64_t*>(read_lane64(reinterpret_cast<int64_t>(mine.a_ptrs), vb.z));
+  P.b_ptrs = reinterpret_cast<const int64_t*>(read_lane64(reinterpret_cast<int64_t>(mine.b_ptrs), vb.z));
+  P.y_offset = read_lane64(mine.y_offset, vb.z);
+  P.y_stride = read_lane64(mine.y_stride, vb.z);
+  P.h_out = read_lane(mine.h_out, vb.z);
   const int h_out = P.h_out;
   constexpr int cols_per_wg = (kBgmvThreads / (R / 8)) * U * NBLK;
   const int col0 = vb.x * cols_per_wg;
