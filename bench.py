@@ -14,13 +14,18 @@ on q/k/v/o): metric/value = tokens x layers per second of the whole step over ex
 "configs" holds the same figures for every configuration; "roofline_min" the lowest HBM-roofline
 fraction of any kernel kind in configurations 1-4.
 
-Per configuration: "ms_per_step" is the median and "ms_per_step_best" the best of several timing
-windows of K steps; "roofline" = algorithmic HBM bytes per launch of the kernel kind that takes
-most of the step divided by its average launch duration, measured with events on the launch
-stream around graphs holding only that kind; "gather_GBps" is the secondary figure that counts an
-adapter's weights once per routed row instead of once per launch (it can exceed the peak through
-cache hits and is never used for the fraction); "cpu_baseline" = the oracle's restatement of the
-reference's per-adapter masked matmul loop timed on the host cores on one layer of the same batch.
+Per configuration: "ms_per_step" is the median of several timing windows of K steps.  "kernels" holds, per
+kernel kind: "n" launches per layer, "MB" algorithmic HBM bytes per launch (10^6 bytes), "us" the average launch
+duration in a graph that holds only that kind, "in_step_us" its duration inside the whole step - (replay time of
+the whole-step graph - replay time of the same graph without that kind) / launches, so a kernel that runs slower
+behind another kind's dirty cache lines is charged for it - and "frac" = MB / in_step_us / 8 TB/s.  All replay
+times come from events recorded on the stream the graphs are launched on.  "roofline" repeats the kind that takes
+most of the step (achieved = MB / in_step_us); "traffic" is the HBM-side bytes per launch from the counter passes
+kept in profiles/traffic.json (not from this run).  "cpu_baseline" = the oracle's restatement of the reference's
+per-adapter masked matmul loop timed on the host cores on one layer of the same batch.
+"ceiling" is what plain torch operations reach in the same process, as graph nodes timed the same way: a
+device-to-device copy of 1 GiB (bytes read + bytes written per second), a copy that moves 32 MiB (16 MiB each
+way, buffers rotated through 512 MiB), and a one-element kernel (the cost of a graph node).
 """
 
 import argparse
@@ -58,6 +63,7 @@ def parse_args():
     p.add_argument("--two-launch", action="store_true",
                    help="fused pattern without the single-launch shrink+expand kernel for ranks 8 and 16")
     p.add_argument("--eager", action="store_true", help="launch every step eagerly instead of replaying a graph")
+    p.add_argument("--no-ceiling", action="store_true", help="skip the plain-torch copy / small-launch measurements")
     return p.parse_args()
 
 
@@ -454,9 +460,67 @@ def cpu_baseline(w, budget_s=5.0):
     }
 
 
+def sig(x, digits=4):
+    """x rounded to `digits` significant digits (keeps the JSON line short)."""
+    if x is None or isinstance(x, (bool, int, str)):
+        return x
+    if x == 0 or x != x:
+        return x
+    from math import floor, log10
+
+    return round(x, digits - 1 - int(floor(log10(abs(x)))))
+
+
+def measure_ceiling(device, reps=10):
+    """What plain torch operations reach on this GPU, as graph nodes timed like the kernels: a 1 GiB copy, a copy
+    that moves 32 MiB, and a one-element kernel."""
+    import torch
+
+    def graph_of(fn, n):
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            fn(0)
+        torch.cuda.current_stream().wait_stream(stream)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(n):
+                fn(i)
+        return g
+
+    big = 1 << 30
+    src = torch.ones(big, dtype=torch.uint8, device=device)
+    dst = torch.empty_like(src)
+    g = graph_of(lambda i: dst.copy_(src), 4)
+    ms, _ = time_graph(g, reps=reps, windows=3)
+    copy_gbps = 2 * big * 4 / (ms * 1e-3) / 1e9
+    del g, src, dst
+    torch.cuda.empty_cache()
+    small = 16 << 20
+    pairs = 16  # 512 MiB of buffers: beyond the 256 MB memory-side cache
+    bufs = torch.ones((2 * pairs, small), dtype=torch.uint8, device=device)
+    g = graph_of(lambda i: bufs[2 * (i % pairs) + 1].copy_(bufs[2 * (i % pairs)]), 4 * pairs)
+    ms, _ = time_graph(g, reps=reps, windows=3)
+    copy32_us = ms * 1e3 / (4 * pairs)
+    del g, bufs
+    torch.cuda.empty_cache()
+    one = torch.zeros(1, dtype=torch.float32, device=device)
+    g = graph_of(lambda i: one.add_(1.0), 200)
+    ms, _ = time_graph(g, reps=reps, windows=3)
+    node_us = ms * 1e3 / 200
+    del g
+    return {
+        "copy_1GiB_GBps": sig(copy_gbps), "copy_1GiB_frac_of_peak": sig(copy_gbps / HBM_PEAK_GBS),
+        "copy_32MiB_moved_us": sig(copy32_us), "copy_32MiB_moved_GBps": sig(2 * small / (copy32_us * 1e-6) / 1e9),
+        "small_launch_us": sig(node_us),
+        "how": "torch copy_/add_ as HIP-graph nodes, events on the launch stream; GB/s = (read + written bytes) / time",
+    }
+
+
 def run_config(cfg: str, args, device):
     """Builds one configuration, times K steps (and further windows of K steps), times every kernel kind on its
-    own, and returns the configuration's record."""
+    own and inside the step, and returns the configuration's record."""
     import torch
 
     w = build_workload(cfg, args.layers, device)
@@ -481,58 +545,72 @@ def run_config(cfg: str, args, device):
         torch.cuda.synchronize()
         window_ms.append((time.perf_counter() - t0) * 1e3 / args.steps)
     first_ms = window_ms[0]  # exactly K steps after W warm-up steps: the figure of the top-level line
-    median_ms, best_ms = statistics.median(window_ms), min(window_ms)
+    median_ms = statistics.median(window_ms)
 
-    # per-kernel timing: graphs that hold only one kind of launch, over the same layer sweep
+    # per-kernel timing over the same layer sweep: graphs that hold only one kind of launch ("us"), and the whole
+    # step without that kind ("in_step_us" = what the kind adds to the step)
     kinds = sorted({c[0] for c in plan.calls if c[0] != "zero"})
+    reps = max(5, min(50, args.steps))
+    windows = max(1, args.windows)
     per_kind = {}
-    for kind in kinds:
-        g, n = capture(plan, L, kinds={kind})
-        ms, ms_best = time_graph(g, reps=max(5, min(50, args.steps)), windows=max(1, args.windows))
-        avg_us = ms * 1e3 / n
-        launches = plan.launches_per_layer(kind)
-        bytes_per_launch = plan.bytes_per_layer(kind) / launches
-        per_kind[kind] = {
-            "launches_per_layer": launches,
-            "avg_launch_us": avg_us,
-            "best_launch_us": ms_best * 1e3 / n,
-            "bytes_per_launch": bytes_per_launch,
-            "GBps": bytes_per_launch / (avg_us * 1e-6) / 1e9,
-            "frac": bytes_per_launch / (avg_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
-            "gather_GBps": plan.gather_bytes_per_layer(kind) / launches / (avg_us * 1e-6) / 1e9,
-            "share_ms": ms,
-        }
-        del g
-    dominant = max(per_kind, key=lambda k: per_kind[k]["share_ms"])
-    dk = per_kind[dominant]
-    traffic = None
+    step_event_ms = None
+    if not args.eager:
+        step_event_ms, _ = time_graph(graph, reps=reps, windows=windows)
+    traffic_all = {}
     traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(traffic_file):
-        traffic = json.load(open(traffic_file)).get(f"cfg{cfg}", {}).get(dominant)
+        traffic_all = json.load(open(traffic_file)).get(f"cfg{cfg}", {})
+    for kind in kinds:
+        g, n = capture(plan, L, kinds={kind})
+        ms, _ = time_graph(g, reps=reps, windows=windows)
+        del g
+        in_step_ms = ms
+        others = {k for k in kinds if k != kind} | ({"zero"} if any(c[0] == "zero" for c in plan.calls) else set())
+        if step_event_ms is not None:
+            if others:
+                g, _ = capture(plan, L, kinds=others)
+                without_ms, _ = time_graph(g, reps=reps, windows=windows)
+                del g
+                in_step_ms = step_event_ms - without_ms
+            else:
+                in_step_ms = step_event_ms
+        launches = plan.launches_per_layer(kind)
+        bytes_per_launch = plan.bytes_per_layer(kind) / launches
+        in_step_us = in_step_ms * 1e3 / n
+        per_kind[kind] = {
+            "n": launches,
+            "MB": bytes_per_launch / 1e6,
+            "us": ms * 1e3 / n,
+            "in_step_us": in_step_us,
+            "GBps": bytes_per_launch / (in_step_us * 1e-6) / 1e9,
+            "frac": bytes_per_launch / (in_step_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "gather_GBps": plan.gather_bytes_per_layer(kind) / launches / (in_step_us * 1e-6) / 1e9,
+            "traffic": traffic_all.get(kind),
+            "share_ms": in_step_ms,
+        }
+    dominant = max(per_kind, key=lambda k: per_kind[k]["share_ms"])
+    dk = per_kind[dominant]
     # A launch whose algorithmic bytes would take less than the ~2 us a graph node costs at the HBM peak is
     # bound by launch latency whatever the kernel does.
-    launch_bound = dk["bytes_per_launch"] / (HBM_PEAK_GBS * 1e9) < 1e-6
+    launch_bound = dk["MB"] * 1e6 / (HBM_PEAK_GBS * 1e9) < 1e-6
 
+    lens = ""
+    if w.prefill:
+        segs = sum(1 for i, a in enumerate(w.adapter_indices) if i == 0 or a != w.adapter_indices[i - 1])
+        lens = f" runs={segs}"
     record = {
-        "workload": w.name,
+        "workload": f"{w.name} T={w.num_tokens}{lens} adapters={w.distinct_adapters()}/{len(w.rank_of_adapter)}",
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f16",
         "value": w.num_tokens * L / (median_ms * 1e-3),
         "unit": "tokens/s per LoRA layer",
         "ms_per_step": median_ms,
-        "ms_per_step_best": best_ms,
         "ms_per_step_first_window": first_ms,
-        "windows": len(window_ms),
         "tokens": w.num_tokens,
-        "routed_tokens": w.routed_tokens(),
-        "distinct_adapters": w.distinct_adapters(),
-        "resident_adapters": len(w.rank_of_adapter),
-        "empty_segments_per_rank_group": len(w.extra_segments) if w.prefill else 0,
         "layers_per_step": L,
-        "projections": [n for g in w.groups for n in g.layer_names],
         "launch": "eager" if args.eager else "hip_graph",
         "pattern": args.pattern,
         "launches_per_layer": plan.launches_per_layer(),
-        "algorithmic_bytes_per_layer": plan.bytes_per_layer(),
+        "MB_per_layer": plan.bytes_per_layer() / 1e6,
         "step_GBps": plan.bytes_per_layer() * L / (median_ms * 1e-3) / 1e9,
         "roofline": {
             "bound": "launch" if launch_bound else "hbm",
@@ -541,11 +619,9 @@ def run_config(cfg: str, args, device):
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": dk["frac"],
-            "traffic": traffic,
-            "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes, not this run)"
-            if traffic is not None else None,
-            "avg_launch_us": dk["avg_launch_us"],
-            "bytes_per_launch": dk["bytes_per_launch"],
+            "traffic": dk["traffic"],
+            "avg_launch_us": dk["in_step_us"],
+            "bytes_per_launch": dk["MB"] * 1e6,
         },
         "kernels": per_kind,
     }
@@ -558,6 +634,25 @@ def run_config(cfg: str, args, device):
         del graph, run_step
     torch.cuda.empty_cache()
     return record
+
+
+def compact(record):
+    """One configuration's record as it goes into the JSON line: 4 significant digits, short keys."""
+    out = {
+        "workload": record["workload"],
+        "dtype": record["dtype"],
+        "value": sig(record["value"]),
+        "ms_per_step": sig(record["ms_per_step"]),
+        "layers": record["layers_per_step"],
+        "launches_per_layer": record["launches_per_layer"],
+        "kernels": {k: {f: sig(v[f]) for f in ("n", "MB", "us", "in_step_us", "frac", "traffic")}
+                    for k, v in record["kernels"].items()},
+        "roofline": {k: sig(v) for k, v in record["roofline"].items() if k not in ("avg_launch_us", "bytes_per_launch")},
+    }
+    cb = record["cpu_baseline"]
+    out["cpu_baseline"] = None if cb is None else {
+        "value": sig(cb["value"]), "cores": cb["cores"], "kind": cb["kind"], "sample": cb["sample"]}
+    return out
 
 
 def main():
@@ -591,41 +686,49 @@ def main():
         print(f"bench: configuration {cfg}", file=sys.stderr, flush=True)
         records[cfg] = run_config(cfg, args, device)
     head = records[todo[0]]  # cfg2 in the default run
+    ceiling = None
+    if not args.eager and not args.no_ceiling:
+        print("bench: ceiling", file=sys.stderr, flush=True)
+        ceiling = measure_ceiling(device)
 
+    cb = head["cpu_baseline"]
     out = {
         "metric": "LoRA-layer tokens/sec (BGMV decode / SGMV prefill), HBM roofline fraction in 'roofline'",
-        "value": head["tokens"] * head["layers_per_step"] / (head["ms_per_step_first_window"] * 1e-3),
+        "value": sig(head["tokens"] * head["layers_per_step"] / (head["ms_per_step_first_window"] * 1e-3), 6),
         "unit": "tokens/s per LoRA layer",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": head["ms_per_step_first_window"],
-        "ms_per_step_median": head["ms_per_step"],
-        "ms_per_step_best": head["ms_per_step_best"],
+        "ms_per_step": sig(head["ms_per_step_first_window"], 6),
+        "ms_per_step_median": sig(head["ms_per_step"], 6),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": head["dtype"],
         "data": "synthetic",
-        "config": {k: head[k] for k in (
-            "workload", "tokens", "routed_tokens", "distinct_adapters", "resident_adapters", "layers_per_step",
-            "projections", "launch", "pattern", "launches_per_layer", "algorithmic_bytes_per_layer", "step_GBps")},
-        "roofline": head["roofline"],
-        "kernels": head["kernels"],
-        "cpu_baseline": head["cpu_baseline"],
+        "config": {"workload": head["workload"], "layers_per_step": head["layers_per_step"], "launch": head["launch"],
+                   "pattern": head["pattern"], "launches_per_layer": head["launches_per_layer"],
+                   "MB_per_layer": sig(head["MB_per_layer"]), "step_GBps": sig(head["step_GBps"])},
+        "roofline": {k: sig(v, 5) for k, v in head["roofline"].items()},
+        "cpu_baseline": None if cb is None else {
+            "value": sig(cb["value"]), "unit": cb["unit"], "cores": cb["cores"], "kind": cb["kind"],
+            "sample": cb["sample"], "cpu_model": cb["cpu_model"], "os_cpu_count": cb["os_cpu_count"]},
+        "ceiling": ceiling,
     }
     if args.config == "all":
-        out["configs"] = {f"cfg{k}": records[k] for k in todo if k not in ("mid", "5dec")}
-        out["extra"] = {"mid_prefill_1k": records["mid"], "cfg5_decode_tokens_bgmv": records["5dec"]}
+        out["configs"] = {f"cfg{k}": compact(records[k]) for k in todo if k not in ("mid", "5dec")}
+        out["extra"] = {"mid_prefill_1k": compact(records["mid"]), "cfg5_decode_tokens_bgmv": compact(records["5dec"])}
         fracs = [(f"cfg{k}", kind, rec["frac"], records[k]["roofline"]["bound"])
                  for k in GATED for kind, rec in records[k]["kernels"].items()]
         lowest = min(fracs, key=lambda t: t[2])
-        out["roofline_min"] = {"config": lowest[0], "kernel": lowest[1], "frac": lowest[2], "bound": lowest[3]}
+        out["roofline_min"] = {"config": lowest[0], "kernel": lowest[1], "frac": sig(lowest[2]), "bound": lowest[3]}
         hbm = [t for t in fracs if t[3] == "hbm"]
         if hbm:
             lowest = min(hbm, key=lambda t: t[2])
-            out["roofline_min_hbm_bound"] = {"config": lowest[0], "kernel": lowest[1], "frac": lowest[2]}
-    print(json.dumps(out))
+            out["roofline_min_hbm_bound"] = {"config": lowest[0], "kernel": lowest[1], "frac": sig(lowest[2])}
+    else:
+        out["kernels"] = compact(head)["kernels"]
+    print(json.dumps(out, separators=(",", ":")))
 
 
 if __name__ == "__main__":

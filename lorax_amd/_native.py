@@ -72,6 +72,7 @@ class TableGroup(ctypes.Structure):
 
 
 MAX_BGMV_PROBLEMS = 16
+MAX_BGMV_TOKENS = 65535  # rows of a BGMV launch and records of one routing plan (capi.hip: bgmv_batch)
 MAX_FUSED_BGMV_PROBLEMS = 4
 
 _SIGNATURES = {

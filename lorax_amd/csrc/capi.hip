@@ -169,12 +169,13 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
 }
 
 // Shape checks and launch shared by lorax_sgmv_shrink and lorax_sgmv_shrink_static.  `scratch_buf` is
-// kShrinkScratchBytes of device memory (partial tiles, then arrival counters) or null.  With `must_fit`, a call
-// that is served by the split-K kernel is refused unless the scratch holds two fp32 partial tiles of the batch.
+// kShrinkScratchBytes of device memory (partial tiles, then arrival counters) or null.  A launch splits the hidden
+// dimension across workgroups only as far as the scratch has room for (sgmv_shrink_ksplit, the K parts of the
+// LDS-staged kernel), so no batch is too large for it.
 int sgmv_shrink_checked(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start, const int32_t* s_end,
                         int32_t num_segments, int64_t num_tokens, int32_t h_in, int32_t r, int32_t a_layout,
-                        int64_t layer_idx, float scale, int32_t accumulate, void* scratch_buf, bool must_fit,
-                        int32_t dtype, void* stream) {
+                        int64_t layer_idx, float scale, int32_t accumulate, void* scratch_buf, int32_t dtype,
+                        void* stream) {
   if (accumulate != 0 && accumulate != 1)
     return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (int rc = check_common(v, x, w_ptrs, dtype)) return rc;
@@ -210,14 +211,6 @@ int sgmv_shrink_checked(void* v, const void* x, const int64_t* w_ptrs, const int
   const ShrinkRoute route = sgmv_shrink_route(a);
   if (route == ShrinkRoute::kNone)
     return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in, r, a_layout);
-  if (must_fit && route == ShrinkRoute::kRegisters) {
-    const int64_t need = 2 * num_tokens * r * static_cast<int64_t>(sizeof(float));
-    if (need > static_cast<int64_t>(kPartialBytes))
-      return fail(LORAX_ESPACE,
-                  "batch too large for the static scratch: 2 * num_tokens * r * 4 = %lld bytes, limit %zu "
-                  "(num_tokens=%lld r=%d); call lorax_sgmv_shrink with a tmp buffer instead",
-                  (long long)need, kPartialBytes, (long long)num_tokens, r);
-  }
   const hipError_t e = launch_sgmv_shrink(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_shrink launch failed: %s", hipGetErrorString(e));
   return LORAX_OK;
@@ -267,7 +260,7 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
   // and its barrier words from tmp).  Its contents are never assumed: the counters are cleared by the launch.
   void* scratch_buf = (a_layout == LORAX_A_RH && aligned16(tmp)) ? tmp : nullptr;
   return sgmv_shrink_checked(v, x, w_ptrs, s_start, s_end, num_segments, num_tokens, h_in, r, a_layout, layer_idx,
-                             scale, 1, scratch_buf, false, dtype, stream);
+                             scale, 1, scratch_buf, dtype, stream);
 }
 
 int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
@@ -286,7 +279,7 @@ int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, cons
   unsigned char* buf = nullptr;
   if (int rc = resolve_scratch(device, &buf)) return rc;
   return sgmv_shrink_checked(v, x, w_ptrs, s_start, s_end, num_segments, num_tokens, h_in, r, a_layout, layer_idx,
-                             scale, 1, buf, true, dtype, stream);
+                             scale, 1, buf, dtype, stream);
 }
 
 int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t num_problems, const void* x,
@@ -314,7 +307,7 @@ int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t
       if (tmp == nullptr) return fail(LORAX_EINVAL, "null pointer argument (tmp)");
       const int rc = sgmv_shrink_checked(problems[i].v, x, problems[i].w_ptrs, s_start, s_end, num_segments, num_tokens,
                                          h_in, r, LORAX_A_RH, layer_idx, scale, accumulate, aligned16(tmp) ? tmp : nullptr,
-                                         false, dtype, stream);
+                                         dtype, stream);
       if (rc != LORAX_OK) return rc;
     }
     return LORAX_OK;
@@ -502,7 +495,20 @@ size_t lorax_sgmv_tmp_size(int32_t num_problems) {
 
 int lorax_init(int32_t device) {
   unsigned char* p = nullptr;
-  return resolve_scratch(device, &p);
+  if (int rc = resolve_scratch(device, &p)) return rc;
+  // Per-kernel attributes (the dynamic LDS limit of the LDS-staged shrink) on that device, so that no launch
+  // has anything left to set up - the first call of every entry point may already be under stream capture.
+  int prev = 0;
+  hipError_t e = hipGetDevice(&prev);
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (prev != device) {
+    e = hipSetDevice(device);
+    if (e != hipSuccess) return fail(LORAX_ELAUNCH, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
+  }
+  e = configure_sgmv_shrink_lds();
+  if (prev != device) (void)hipSetDevice(prev);
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "kernel set-up on device %d: %s", device, hipGetErrorString(e));
+  return LORAX_OK;
 }
 
 size_t lorax_workspace_bytes(void) { return kShrinkScratchBytes; }

@@ -157,6 +157,9 @@ hipError_t launch_sgmv_expand_t(const SgmvArgs& a, hipStream_t stream);  // B st
 // LDS-staged shrink (sgmv_shrink_lds.hip): [L, r, h_in] layout, h_in a multiple of 128.
 bool sgmv_shrink_lds_applies(const SgmvArgs& a);
 hipError_t launch_sgmv_shrink_lds(const SgmvArgs& a, hipStream_t stream);
+// Per-device set-up of the LDS-staged shrink on the current device (the dynamic LDS limit of every instantiation),
+// so that no launch has first-call state; a launch that finds it missing does it itself.
+hipError_t configure_sgmv_shrink_lds();
 // Streaming shrink for a handful of rows (bgmv.hip): [L, r, h_in] layout, any h_in the BGMV kernels take.
 hipError_t launch_sgmv_shrink_rows(const SgmvArgs& a, hipStream_t stream);
 
@@ -165,9 +168,10 @@ hipError_t launch_sgmv_shrink_rows(const SgmvArgs& a, hipStream_t stream);
 enum class ShrinkRoute {
   kNone,       // no kernel takes the shape
   kRows,       // streaming kernel for a few hundred rows, [L, r, h_in]
-  kLds,        // LDS-staged MFMA kernel, [L, r, h_in], h_in a multiple of 128
-  kRegisters,  // register-operand MFMA kernel, [L, r, h_in], r a multiple of 16; the only one that may split K
-               // across workgroups and so the only one that touches the scratch
+  kLds,        // LDS-staged MFMA kernel, [L, r, h_in], h_in a multiple of 128; launches of few row tiles cut K
+               // into parts and keep the parts' fp32 sums in the scratch
+  kRegisters,  // register-operand MFMA kernel, [L, r, h_in], r a multiple of 16; may split K across workgroups
+               // (fp32 partial tiles and arrival counters in the scratch)
   kNarrowRows  // [L, h_in, r] layout (rank 8 in the reference)
 };
 ShrinkRoute sgmv_shrink_route(const SgmvArgs& a);

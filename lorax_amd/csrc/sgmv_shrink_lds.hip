@@ -287,6 +287,21 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_parts_kernel(
 // ---------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------
+// Raising the dynamic LDS limit is needed once per kernel instantiation and device (the current one).
+template <typename D, int NB, int MBLK, bool KSPLIT>
+static hipError_t raise_lds_limit() {
+  static std::atomic<bool> configured[64] = {};  // callers may come from several host threads
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  if (device >= 0 && device < 64 && configured[device].load(std::memory_order_acquire)) return hipSuccess;
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(sgmv_shrink_lds_kernel<D, NB, MBLK, KSPLIT>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMaxBytes);
+  if (e != hipSuccess) return e;
+  if (device >= 0 && device < 64) configured[device].store(true, std::memory_order_release);
+  return hipSuccess;
+}
+
 template <typename D, int NB, int MBLK, bool KSPLIT>
 static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_rows = 0) {
   constexpr int kStageBytes = (MBLK + NB) * 16 * kLdsRowBytes;
@@ -353,17 +368,8 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_
   int lds_bytes = stages * kStageBytes;
   if (lds_bytes < kRedBytes) lds_bytes = kRedBytes;
   auto kernel = sgmv_shrink_lds_kernel<D, NB, MBLK, KSPLIT>;
-  // Raising the dynamic LDS limit is needed once per kernel and device.
-  static std::atomic<bool> configured[64] = {};  // callers may come from several host threads
-  int device = 0;
-  hipError_t e = hipGetDevice(&device);
-  if (e != hipSuccess) return e;
-  if (device < 0 || device >= 64 || !configured[device].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kLdsMaxBytes);
-    if (e != hipSuccess) return e;
-    if (device >= 0 && device < 64) configured[device].store(true, std::memory_order_release);
-  }
+  // lorax_init has raised the dynamic LDS limit of every instantiation; a caller that skipped it gets it here.
+  if (hipError_t e = raise_lds_limit<D, NB, MBLK, KSPLIT>(); e != hipSuccess) return e;
   dim3 grid(static_cast<unsigned>(kparts > 1 ? wgs : (tiles < (1 << 20) ? tiles : (1 << 20))));
   ShrinkGroup grp = a.group;
   if (grp.count <= 1) {
@@ -377,7 +383,7 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_
                      a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages,
                      a.scale, a.accumulate, rows_per_tile, kparts, static_cast<int>(tiles), a.partials,
                      tuning().shrink_no_rotate ? 0 : 1);
-  e = hipGetLastError();
+  const hipError_t e = hipGetLastError();
   if (e != hipSuccess || kparts == 1) return e;
   hipLaunchKernelGGL(sgmv_shrink_parts_kernel<D>, dim3(static_cast<unsigned>(tiles)), dim3(kLdsThreads), 0, stream, grp,
                      a.partials, a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), R, kparts, a.scale,
@@ -435,6 +441,42 @@ static hipError_t launch_lds_dtype(const SgmvArgs& a, hipStream_t stream) {
     default:
       return hipErrorInvalidValue;
   }
+}
+
+// Every instantiation launch_lds_nb can reach, for the per-device set-up: the same case analysis as the launchers.
+template <typename D, int NB>
+static hipError_t raise_lds_limits_nb() {
+  hipError_t e = hipSuccess;
+  auto also = [&](hipError_t r) { if (e == hipSuccess) e = r; };
+  if constexpr (NB <= 4) {
+    also(raise_lds_limit<D, NB, 4, true>());
+    also(raise_lds_limit<D, NB, 3, true>());
+  }
+  also(raise_lds_limit<D, NB, 4, false>());
+  if constexpr (NB > 4) also(raise_lds_limit<D, NB, 3, true>());
+  else if constexpr (NB % 4 == 0) also(raise_lds_limit<D, NB, 3, false>());
+  if constexpr (NB % 2 == 0) also(raise_lds_limit<D, NB, 2, false>());
+  also(raise_lds_limit<D, NB, 2, true>());
+  also(raise_lds_limit<D, NB, 1, true>());
+  return e;
+}
+template <typename D>
+static hipError_t raise_lds_limits_dtype() {
+  hipError_t e = hipSuccess;
+  auto also = [&](hipError_t r) { if (e == hipSuccess) e = r; };
+  also(raise_lds_limits_nb<D, 1>());
+  also(raise_lds_limits_nb<D, 2>());
+  also(raise_lds_limits_nb<D, 3>());
+  also(raise_lds_limits_nb<D, 4>());
+  also(raise_lds_limits_nb<D, 5>());
+  also(raise_lds_limits_nb<D, 6>());
+  also(raise_lds_limits_nb<D, 7>());
+  also(raise_lds_limits_nb<D, 8>());
+  return e;
+}
+hipError_t configure_sgmv_shrink_lds() {
+  const hipError_t e = raise_lds_limits_dtype<F16>();
+  return e != hipSuccess ? e : raise_lds_limits_dtype<BF16>();
 }
 
 bool sgmv_shrink_lds_applies(const SgmvArgs& a) {

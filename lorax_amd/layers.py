@@ -173,7 +173,10 @@ class LoraLinear(nn.Module):
             # can, and once for up to four rows.  Both write disjoint rows of v and of the result.
             first = group[0][0]
             plans = [rs.short_plan for rs, _, _ in group]
-            split = all(p is not None for p in plans)
+            # (the per-token kernels number rows and plan records with 16 bits; beyond that the segment kernels
+            # take the whole tables, which still list every segment)
+            split = (all(p is not None for p in plans) and input.size(0) <= _native.MAX_BGMV_TOKENS
+                     and all(p.size(0) <= _native.MAX_BGMV_TOKENS for p in plans))
             n_long = first.num_long_segments if split else first.segment_starts.numel()
             starts, ends = first.segment_starts[:n_long], first.segment_ends[:n_long]
             # v needs no zero-fill: the shrinks overwrite the rows of their segments and the expands read no others

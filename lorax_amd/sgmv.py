@@ -89,22 +89,26 @@ def orient_for_rank(t: torch.Tensor, rank: int) -> torch.Tensor:
     return t.transpose(0, 1) if MIN_RANK_CUSTOM <= rank <= MAX_RANK_CUSTOM else t
 
 
-@lru_cache(maxsize=1)
+_tmp_tensors = {}  # device -> the 8 MiB scratch, one per device for the life of the process
+
+
 def get_tmp_tensor(device: torch.device) -> torch.Tensor:
-    """punica.py:145-147."""
-    return torch.empty((_SHRINK_TMP_BYTES,), dtype=torch.uint8, device=device)
+    """punica.py:145-147 (cached per device: callers that alternate between devices keep both buffers)."""
+    device = torch.device(device)
+    if device.type == "cuda" and device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    tmp = _tmp_tensors.get(device)
+    if tmp is None:
+        tmp = _tmp_tensors[device] = torch.empty((_SHRINK_TMP_BYTES,), dtype=torch.uint8, device=device)
+    return tmp
 
 
-_RESIDENT_SCRATCH_BYTES = 32 * 1024 * 1024
-
-
-@lru_cache(maxsize=1)
 def get_shrink_scratch(device: torch.device) -> torch.Tensor:
     """Scratch of the resident-layout shrink entries (lora_a_sgmv_resident, lora_a_sgmv_resident_multi): where a
-    batch has fewer row tiles than the GPU has CUs, K is split across workgroups and the fp32 partial sums
-    (splits x rows x summed rank) go here.  The reference's 8 MiB buffer (get_tmp_tensor) is accepted too and
-    only limits how far such a launch can split."""
-    return torch.empty((_RESIDENT_SCRATCH_BYTES,), dtype=torch.uint8, device=device)
+    batch has fewer row tiles than the GPU has CUs, the hidden dimension is cut into parts across workgroups and
+    the parts' fp32 sums (parts x rows x summed rank) go here.  It is the reference's 8 MiB buffer: the kernels
+    keep their sums inside the first 8 MiB whatever a caller passes, so that the result does not depend on it."""
+    return get_tmp_tensor(device)
 
 
 def get_tmp_expand_size(size: int) -> int:

@@ -499,3 +499,44 @@ def test_native_table_builder_reports_the_space_it_needs():
     assert g8.use_sgmv == 1 and g8.num_segments == 2 and g8.plan_off == -1
     assert packed.view(np.int32)[g8.starts_off // 4 : g8.starts_off // 4 + 2].tolist() == [0, 4]
     assert packed.view(np.int32)[g8.ends_off // 4 : g8.ends_off // 4 + 2].tolist() == [2, 5]
+
+
+def test_prefill_batches_beyond_the_per_token_kernels_range_stay_on_the_segment_kernels(monkeypatch):
+    """The per-token kernels number rows and plan records with 16 bits.  A prefill batch whose short segments have
+    a routing plan goes to them only inside that range; beyond it the segment kernels take the complete tables,
+    which still list every segment (the limit is lowered here so that a small batch crosses it)."""
+    from lorax_amd import _native, layers
+    from lorax_amd.adapters import LORA, AdapterBatchData, BatchLoraWeights, LayerAdapterWeights, LoraConfig, LoraWeights
+    from lorax_amd.synthetic import make_meta
+
+    h, L, r = 128, 1, 32  # rank 32: outside the single-launch prefill update
+    layer = LayerAdapterWeights()
+    for idx in range(6):
+        layer.add_adapter(idx, LoraWeights([torch.randn(h, r)] * L, [torch.randn(r, h)] * L, LoraConfig(r=r)))
+    idx = [0] * 40
+    for i in range(40):
+        idx += [1 + i % 5] * (1 + i % 3) + [-1]
+    meta = make_meta(idx, torch.device("cpu"))
+    batch = BatchLoraWeights.load(layer.adapter_weights, meta, "q_proj", True, None)
+    rd = batch.rank_data[r]
+    assert rd.short_plan is not None and rd.num_long_segments == 1
+    data = AdapterBatchData(meta=meta, data={"q_proj": {LORA: batch}}, layer_to_lora_weights={}, punica_wrapper=None,
+                            prefill=True)
+    calls = []
+    monkeypatch.setattr(layers, "has_sgmv", lambda: True)
+    monkeypatch.setattr(layers, "get_shrink_scratch", lambda device: None)
+    monkeypatch.setattr(layers, "get_tmp_expand_size", lambda n: 60 * n)
+    monkeypatch.setattr(_native, "sgmv_shrink_multi", lambda vs, x, tables, s, e, *a, **k: calls.append(("shrink", s.numel())))
+    monkeypatch.setattr(_native, "bgmv_multi", lambda *a, **k: calls.append(("bgmv", None)))
+    monkeypatch.setattr(layers, "lora_b_sgmv_cutlass_slice",
+                        lambda y, v, tmp, table, s, e, *a, **k: calls.append(("expand", s.numel())))
+    lin = layers.LoraLinear(None, 0)
+    x = torch.zeros((len(idx), h), dtype=torch.bfloat16)
+    y = torch.zeros((len(idx), h), dtype=torch.bfloat16)
+    lin.forward_layer_type(y, x, data, "q_proj", 0, h)
+    assert calls == [("shrink", 1), ("bgmv", None), ("expand", 1), ("bgmv", None)]  # inside the range: split
+    calls.clear()
+    monkeypatch.setattr(_native, "MAX_BGMV_TOKENS", len(idx) - 1)
+    lin.forward_layer_type(y, x, data, "q_proj", 0, h)
+    n_all = rd.segment_starts.numel()
+    assert calls == [("shrink", n_all), ("expand", n_all)]  # beyond it: every segment on the segment kernels

@@ -32,11 +32,15 @@ def _both(r, h_in, lens, seed, layer=1):
     v_ref = torch.zeros((x.size(0), r), dtype=x.dtype, device=DEV)
     _native.sgmv_shrink(v_ref, x, table, s_start, s_end, tmp, layer)
     v = torch.zeros_like(v_ref)
+    _native.init(torch.device(DEV))  # the per-device set-up; after it the entry point has nothing left to set up
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # free device memory as the driver reports it: a hipMalloc inside the library would show here, whoever made it
+    # (torch's own counter only sees torch's allocator)
+    free_before, allocated_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
     _native.sgmv_shrink_static(v, x, table, s_start, s_end, layer)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.cuda.memory_allocated() == allocated_before
     want = torch.zeros((x.size(0), r), dtype=x.dtype)
     for i, (s, e) in enumerate(zip(starts, ends)):
         if e > s:
@@ -59,18 +63,3 @@ def test_static_shrink_matches_the_tmp_entry_point(r, h_in, first, second):
         assert_close(v, want, f"v lens={lens}")
 
 
-def test_static_shrink_refuses_batches_beyond_its_scratch():
-    r, h_in, T = 128, 1056, 8200  # 2 * 8200 * 128 * 4 bytes exceed the scratch; h_in is not a multiple of 128
-    x = torch.zeros((T, h_in), dtype=torch.bfloat16, device=DEV)
-    v = torch.zeros((T, r), dtype=torch.bfloat16, device=DEV)
-    w = torch.zeros((1, r, h_in), dtype=torch.bfloat16, device=DEV)
-    s_start = torch.tensor([0], dtype=torch.int32, device=DEV)
-    s_end = torch.tensor([T], dtype=torch.int32, device=DEV)
-    with pytest.raises(RuntimeError, match="static scratch"):
-        _native.sgmv_shrink_static(v, x, ptr_table([w], DEV), s_start, s_end, 0)
-    # the same batch through the LDS-staged kernel (h_in a multiple of 128) needs no scratch and is served
-    x2 = torch.ones((T, 1024), dtype=torch.bfloat16, device=DEV)
-    w2 = torch.ones((1, r, 1024), dtype=torch.bfloat16, device=DEV)
-    _native.sgmv_shrink_static(v, x2, ptr_table([w2], DEV), s_start, s_end, 0)
-    torch.cuda.synchronize()
-    assert torch.all(v == 1024)
