@@ -63,6 +63,8 @@ def parse_args():
     p.add_argument("--two-launch", action="store_true",
                    help="fused pattern without the single-launch shrink+expand kernel for ranks 8 and 16")
     p.add_argument("--eager", action="store_true", help="launch every step eagerly instead of replaying a graph")
+    p.add_argument("--no-tiles", action="store_true",
+                   help="prefill launches search their row tiles on the device instead of taking the tables' plans")
     p.add_argument("--no-ceiling", action="store_true", help="skip the plain-torch copy / small-launch measurements")
     return p.parse_args()
 
@@ -95,7 +97,7 @@ class Plan:
     caller's sequence (utils/layers.py:114-164): zero-fill, shrink, expand for every projection and rank.
     """
 
-    def __init__(self, w, pattern="fused", use_plan=True, fuse_small_ranks=True):
+    def __init__(self, w, pattern="fused", use_plan=True, fuse_small_ranks=True, use_tiles=True):
         import torch
 
         from lorax_amd import _native
@@ -105,6 +107,7 @@ class Plan:
         self.pattern = pattern
         self.use_plan = use_plan
         self.fuse_small_ranks = fuse_small_ranks
+        self.use_tiles = use_tiles  # prefill launches take the tables' host-built row-tile plans
         self.batch = w.batch_data()
         self.calls = []  # (kind, fn(layer), algorithmic bytes, flops, gather bytes: weights once per routed row)
         T = w.num_tokens
@@ -182,9 +185,13 @@ class Plan:
         if a_is_rh:
             tmp_s = sgmv.get_shrink_scratch(x.device) if resident_a else sgmv.get_tmp_tensor(x.device)
 
+        whole = rd.num_long_segments == starts.numel()  # the tables' row-tile plans cover the long segments
+        shrink_tiles = rd.shrink_tiles if (fused and whole and self.use_tiles) else None
+        expand_tiles = rd.expand_tiles if (fused and whole and self.use_tiles) else None
+
         def shrink(layer):
             if resident_a:  # overwrites the segments' rows of v: no zero-fill in this pattern
-                sgmv._kernels.sgmv_shrink_multi([v], x, [a_ptr], starts, ends, tmp_s, layer, 1.0, False)
+                sgmv._kernels.sgmv_shrink_multi([v], x, [a_ptr], starts, ends, tmp_s, layer, 1.0, False, shrink_tiles)
             elif a_is_rh:
                 sgmv._kernels.sgmv_shrink(v, x, a_ptr, starts, ends, tmp_s, layer)
             else:
@@ -192,7 +199,8 @@ class Plan:
 
         def expand(layer):
             if bt_ptr is not None:
-                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, bt_ptr, starts, ends, layer, off, size, transposed=True)
+                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, bt_ptr, starts, ends, layer, off, size, transposed=True,
+                                               tiles=expand_tiles)
             else:
                 sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_ptr, starts, ends, layer, off, size)
 
@@ -219,6 +227,9 @@ class Plan:
         split = all(p is not None for p in plans)
         n_long = first.num_long_segments if split else first.segment_starts.numel()
         starts, ends = first.segment_starts[:n_long], first.segment_ends[:n_long]
+        planned = self.use_tiles and n_long == first.num_long_segments
+        shrink_tiles = first.shrink_tiles if planned else None
+        expand_tiles = first.expand_tiles if planned else None
         lens = (ends - starts).clamp(min=0)
         rows = int(lens.sum().item())
         flat = torch.zeros((len(jobs), x.size(0), r), dtype=x.dtype, device=x.device)
@@ -233,7 +244,7 @@ class Plan:
                 shrink_gather += rows * r * h_in * e + rows * r * e
 
             def shrink(layer, out=vs[i:i + step], tables=tables):
-                _native.sgmv_shrink_multi(out, x, tables, starts, ends, tmp_s, layer, 1.0, False)
+                _native.sgmv_shrink_multi(out, x, tables, starts, ends, tmp_s, layer, 1.0, False, shrink_tiles)
 
             self.calls.append(("sgmv_shrink", shrink, shrink_bytes, 2 * rows * r * h_in * len(tables), shrink_gather))
         if split:
@@ -252,7 +263,8 @@ class Plan:
             uniq = len(set(b_table[lens > 0].tolist()))
 
             def expand(layer, v=v, b_table=b_table, tmp_e=tmp_e, off=off, size=size):
-                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_table, starts, ends, layer, off, size, transposed=True)
+                sgmv.lora_b_sgmv_cutlass_slice(y, v, tmp_e, b_table, starts, ends, layer, off, size, transposed=True,
+                                               tiles=expand_tiles)
 
             self.calls.append(("sgmv_expand", expand, rows * r * e + uniq * r * size * e + 2 * rows * size * e,
                                2 * rows * r * size, rows * r * e + rows * r * size * e + 2 * rows * size * e))
@@ -525,7 +537,7 @@ def run_config(cfg: str, args, device):
 
     w = build_workload(cfg, args.layers, device)
     L = w.num_layers
-    plan = Plan(w, args.pattern, not args.no_plan, not args.two_launch)
+    plan = Plan(w, args.pattern, not args.no_plan, not args.two_launch, not args.no_tiles)
     torch.cuda.synchronize()
 
     if args.eager:

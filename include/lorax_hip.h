@@ -174,23 +174,68 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
 /*
  * lorax_sgmv_shrink without a tmp argument and without any allocation.  It has no counterpart in the reference;
  * it is for callers that cannot allocate device memory or hand a scratch buffer over: code under HIP graph
- * capture, tight serving loops, harnesses that forbid hipMalloc.  The result is bit-identical to
- * lorax_sgmv_shrink's on the same arguments.  The split-K scratch is an array of LORAX_SHRINK_TMP_BYTES (8 MiB)
- * inside the library's own device image, one copy per GPU, held until the process ends; its address on a
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Whenever it returns LORAX_OK the result is
+ * bit-identical to lorax_sgmv_shrink's on the same arguments.  The scratch is an array of LORAX_SHRINK_TMP_BYTES
+ * (8 MiB) inside the library's own device image, one copy per GPU, held until the process ends; its address on a
  * device is looked up on the first call there (or by lorax_init).
  *
- * Limit: a call served by the register-operand kernel (LORAX_A_RH, h_in not a multiple of 128, more than 512
- * rows) needs 2 * num_tokens * r * 4 bytes <= LORAX_SHRINK_TMP_BYTES - 65536, i.e. room for two fp32 partial
- * tiles of the batch; beyond that the call fails with LORAX_ESPACE and launches nothing.  Other shapes have no
- * limit: they use no scratch, or (h_in a multiple of 128, about 500 to 2000 rows) split the hidden dimension
- * only as far as the array has room for.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
- * streams or threads) race; calls on one stream, or ordered by events, do not.  Nothing needs to be cleared
- * between calls (the arrival counters are cleared by every launch that uses them).
+ * Limit: a launch that splits the hidden dimension across workgroups (batches of fewer than 192 row tiles, i.e.
+ * up to a few thousand rows) keeps one fp32 copy of v per part in the array, and all parts of the split the
+ * launcher chooses for the shape must fit: parts * num_tokens * 16 * ceil(r / 16) * 4 bytes <= 8 MiB - 64 KiB.
+ * A call beyond that fails with LORAX_ESPACE and launches nothing (lorax_sgmv_shrink runs the same call with a
+ * shallower split, which is slower; here that never happens silently).  In practice only shapes served by the
+ * register-operand kernel (h_in not a multiple of 128) with around ten thousand rows reach the limit; calls that
+ * do not split - most - use no scratch and have no limit.  All calls on one GPU share that GPU's array: calls
+ * that overlap in time on one GPU (different streams or threads) race; calls on one stream, or ordered by events,
+ * do not.  Nothing needs to be cleared between calls (the arrival counters are cleared by every launch that uses
+ * them, partial sums are written before they are read).
  */
 int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
                              const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t h_in,
                              int32_t r, int32_t a_layout, int64_t layer_idx, float scale, int32_t dtype,
                              void* stream);
+
+/*
+ * Row-tile plan of an SGMV launch (optional; no counterpart in the reference's custom shrink, which searches its
+ * tiles on the device, sgmv_flashinfer.cuh:41-60; its cutlass path precomputes a problem table on the device,
+ * sgmv/sgmv_cutlass.cuh:30-52).  The segment kernels cut every segment into row tiles.  Given only s_start / s_end in device
+ * memory, every workgroup finds its tile by scanning those tables and the grid is sized for an upper bound of the
+ * tile count.  A caller that knows the segment lengths on the host can pass the finished list instead:
+ * `tiles` points to num_tiles records in DEVICE memory, each rows [row0, row_end) of segment `seg` (an index into
+ * the call's s_start / s_end / w_ptrs tables; row0 >= s_start[seg], row_end <= s_end[seg]), `index` the tile's
+ * number inside its segment.  Every row of every non-empty segment must be in exactly one tile, and no tile may
+ * be higher than tile_rows.  lorax_sgmv_plan_tiles builds such a list from host copies of the tables (and
+ * lorax_build_batch_tables emits one per rank group).  Records are clamped on the device to the call's
+ * num_segments, num_tokens and tile_rows, so a wrong plan gives wrong results but touches no memory outside the
+ * call's tensors.  The results do not depend on how a batch is cut into tiles, except that the shrink's last
+ * rounding can (its sums over the hidden dimension are added in an order that depends on the tile, see
+ * lorax_sgmv_shrink_multi).
+ */
+typedef struct lorax_sgmv_tile {
+  int32_t seg;
+  int32_t row0;
+  int32_t row_end;
+  int32_t index;
+} lorax_sgmv_tile_t;
+
+typedef struct lorax_sgmv_tiles {
+  const lorax_sgmv_tile_t* tiles; /* device memory, 16-byte aligned */
+  int32_t num_tiles;
+  int32_t tile_rows;              /* upper bound of row_end - row0 over the list */
+} lorax_sgmv_tiles_t;
+
+#define LORAX_TILES_SHRINK 0 /* for lorax_sgmv_shrink_multi: tiles of at most 64 rows                    */
+#define LORAX_TILES_EXPAND 1 /* for lorax_sgmv_expand_planned: tiles of about 256 rows                   */
+
+/*
+ * Builds a tile plan on the HOST: s_start / s_end are host copies of the segment tables of the launch (empty and
+ * negative segments get no tile, bounds are clamped to [0, num_tokens]).  Writes up to `capacity` records to
+ * `tiles` (host memory; the caller uploads them), the number of records to *num_tiles and the bound of their
+ * heights to *tile_rows.  Returns LORAX_ESPACE, with *num_tiles set, when capacity is too small (or tiles NULL).
+ */
+int lorax_sgmv_plan_tiles(const int32_t* s_start, const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
+                          int32_t kind, lorax_sgmv_tile_t* tiles, int32_t capacity, int32_t* num_tiles,
+                          int32_t* tile_rows);
 
 /*
  * SGMV shrink of up to 4 projections that share x, the segments and the rank (q/k/v, gate/up), LORAX_A_RH
@@ -206,6 +251,15 @@ int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, cons
  * accumulate = 1 adds to v as lorax_sgmv_shrink does; accumulate = 0 stores dtype(scale * x @ A^T) into the rows
  * of the segments instead, so the caller need not zero v first (rows outside every segment keep their contents;
  * lorax_sgmv_expand reads no others).  The reference zero-fills v before every shrink (punica.py:176-178).
+ * `tiles`: optional row-tile plan (LORAX_TILES_SHRINK) for the call's segment tables, or NULL; it is used by the
+ * one-launch path and ignored otherwise.
+ * Order of the sums: a row tile walks the hidden dimension from a starting point that depends on the tile (its
+ * adapter's stack address, its number inside the segment, the XCD it runs on), and launches with few tiles cut
+ * the hidden dimension into parts whose fp32 sums are added afterwards.  A call is deterministic, but the last
+ * rounding of an element of v can differ between two batches that hold the same row (within the parity
+ * tolerance by a wide margin: one spacing of dtype on a few percent of the elements).
+ * lorax_set_fixed_order_shrink(1) gives that up for speed: every tile then walks from k = 0 and no launch cuts
+ * the hidden dimension, so a row's result depends on nothing but the row and its adapter.
  */
 typedef struct {
   void* v;               /* [num_tokens, r] */
@@ -215,7 +269,13 @@ typedef struct {
 int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t num_problems, const void* x,
                             const int32_t* s_start, const int32_t* s_end, int32_t num_segments,
                             int64_t num_tokens, int32_t h_in, int32_t r, int64_t layer_idx, float scale,
-                            int32_t accumulate, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream);
+                            int32_t accumulate, void* tmp, int64_t tmp_bytes, const lorax_sgmv_tiles_t* tiles,
+                            int32_t dtype, void* stream);
+
+/* Process-wide switch (default 0): 1 = the SGMV shrinks add their sums over the hidden dimension in one fixed
+ * order whatever the batch (see lorax_sgmv_shrink_multi).  Returns the previous value.  Not meant to be flipped
+ * while launches are being issued from other threads. */
+int lorax_set_fixed_order_shrink(int32_t on);
 
 /*
  * Shrink and expand of a SHORT prefill batch in one launch, for up to 4 projections that share x and the
@@ -261,6 +321,16 @@ int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32
                       int64_t layer_idx, int32_t accumulate, void* tmp, int64_t tmp_bytes,
                       int32_t dtype, void* stream);
 
+/*
+ * lorax_sgmv_expand over B^T stacks (LORAX_B_HR) with a row-tile plan (LORAX_TILES_EXPAND) and without the tmp
+ * argument, which that kernel has no use for.  No counterpart in the reference.  Same result as lorax_sgmv_expand,
+ * bit for bit (every element of the update is one dot product over r whatever the tiling); `tiles` may be NULL.
+ */
+int lorax_sgmv_expand_planned(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
+                              const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
+                              int32_t h_out, int64_t y_offset, int64_t y_stride, int64_t layer_idx,
+                              int32_t accumulate, const lorax_sgmv_tiles_t* tiles, int32_t dtype, void* stream);
+
 /* Bytes of grouped-GEMM argument scratch for `num_problems` segments.  Replaces
  * sgmv_tmp_size (sgmv/sgmv_cutlass.cuh:54-58): 3 pointers + 3 int64 + one
  * 3 x int32 problem size per segment = 60 * num_problems. */
@@ -287,6 +357,8 @@ size_t lorax_sgmv_tmp_size(int32_t num_problems);
  *   num_long_segments entries and lorax_bgmv_multi over the plan, on the same v and y, instead of the segment
  *   kernels over the whole table.  The reference routes every row of such a batch through its segment kernels
  *   (lorax_server/adapters/lora.py:279, server/lorax_server/models/flash_causal_lm.py:1594).
+ * Every segment-table group also carries the row-tile plans of its first num_long_segments segments for
+ *   lorax_sgmv_shrink_multi and lorax_sgmv_expand_planned (the builder has the segment lengths anyway).
  */
 typedef struct lorax_adapter_entry {
   int64_t adapter; /* adapter index as it appears in adapter_indices            */
@@ -311,6 +383,14 @@ typedef struct lorax_table_group {
   int64_t ends_off;
   int64_t indices_off;  /* int64[num_tokens] slot in the group's tables or -1 (use_sgmv = 0) */
   int64_t plan_off;     /* int64[num_chunks][8] routing plan, -1 = none                   */
+  /* use_sgmv = 1: row-tile plans over the first num_long_segments entries of the tables (lorax_sgmv_tile_t
+     records at these offsets; -1 = none) */
+  int64_t shrink_tiles_off;
+  int64_t expand_tiles_off;
+  int32_t num_shrink_tiles;
+  int32_t shrink_tile_rows;
+  int32_t num_expand_tiles;
+  int32_t expand_tile_rows;
 } lorax_table_group_t;
 
 int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t num_tokens,

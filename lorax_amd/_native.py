@@ -18,6 +18,7 @@ import torch  # noqa: F401  (must be imported first so that its HIP runtime is t
 LIB_PATH = Path(__file__).resolve().parent / "liblorax_hip.so"
 
 F16, BF16 = 0, 1
+ESPACE = 5
 A_RH, A_HR = 0, 1
 B_RH, B_HR = 0, 1
 SHRINK_TMP_BYTES = 8 * 1024 * 1024
@@ -68,7 +69,40 @@ class TableGroup(ctypes.Structure):
     _fields_ = [("layer_type", _c.c_int32), ("rank", _c.c_int32), ("use_sgmv", _c.c_int32),
                 ("num_segments", _c.c_int32), ("num_chunks", _c.c_int32), ("num_long_segments", _c.c_int32),
                 ("a_ptr_off", _c.c_int64), ("b_ptr_off", _c.c_int64), ("starts_off", _c.c_int64),
-                ("ends_off", _c.c_int64), ("indices_off", _c.c_int64), ("plan_off", _c.c_int64)]
+                ("ends_off", _c.c_int64), ("indices_off", _c.c_int64), ("plan_off", _c.c_int64),
+                ("shrink_tiles_off", _c.c_int64), ("expand_tiles_off", _c.c_int64),
+                ("num_shrink_tiles", _c.c_int32), ("shrink_tile_rows", _c.c_int32),
+                ("num_expand_tiles", _c.c_int32), ("expand_tile_rows", _c.c_int32)]
+
+
+class SgmvTiles(ctypes.Structure):
+    """lorax_sgmv_tiles_t of include/lorax_hip.h."""
+
+    _fields_ = [("tiles", _c.c_void_p), ("num_tiles", _c.c_int32), ("tile_rows", _c.c_int32)]
+
+
+TILES_SHRINK, TILES_EXPAND = 0, 1
+
+
+class TilePlan:
+    """A row-tile plan of an SGMV launch: `records` is an int32 [num_tiles, 4] tensor on the launch's device
+    (seg, row0, row_end, index per tile), `tile_rows` the bound of the tiles' heights."""
+
+    __slots__ = ("records", "num_tiles", "tile_rows")
+
+    def __init__(self, records: torch.Tensor, tile_rows: int):
+        if records.dtype != torch.int32 or records.dim() != 2 or records.size(1) != 4 or not records.is_contiguous():
+            raise RuntimeError("tile records must be a contiguous int32 [num_tiles, 4] tensor")
+        self.records = records
+        self.num_tiles = records.size(0)
+        self.tile_rows = int(tile_rows)
+
+    def c_struct(self, device) -> "SgmvTiles":
+        if self.records.device != device:
+            raise RuntimeError(f"tile plan on {self.records.device}, launch on {device}")
+        # (a plan without tiles has no storage; any non-null address marks it as a plan)
+        addr = self.records.data_ptr() if self.num_tiles > 0 else 16
+        return SgmvTiles(addr, self.num_tiles, self.tile_rows)
 
 
 MAX_BGMV_PROBLEMS = 16
@@ -105,9 +139,20 @@ _SIGNATURES = {
     "lorax_sgmv_shrink_multi": (
         _c.c_int,
         [_c.POINTER(SgmvShrinkProblem), _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
-         _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_int32, _c.c_void_p, _c.c_int64, _c.c_int32,
-         _c.c_void_p],
+         _c.c_int32, _c.c_int32, _c.c_int64, _c.c_float, _c.c_int32, _c.c_void_p, _c.c_int64, _c.POINTER(SgmvTiles),
+         _c.c_int32, _c.c_void_p],
     ),
+    "lorax_sgmv_expand_planned": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64, _c.c_int32,
+         _c.c_int32, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int32, _c.POINTER(SgmvTiles), _c.c_int32, _c.c_void_p],
+    ),
+    "lorax_sgmv_plan_tiles": (
+        _c.c_int,
+        [_c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64, _c.c_int32, _c.c_void_p, _c.c_int32,
+         _c.POINTER(_c.c_int32), _c.POINTER(_c.c_int32)],
+    ),
+    "lorax_set_fixed_order_shrink": (_c.c_int, [_c.c_int32]),
     "lorax_sgmv_lora_multi": (
         _c.c_int,
         [_c.POINTER(SgmvLoraProblem), _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64,
@@ -381,11 +426,23 @@ def _check_sgmv(y, x, w_ptr, s_start, s_end, tmp) -> None:
 
 
 def sgmv_expand(y, x, w_ptr, s_start, s_end, tmp, layer_idx, y_offset=0, y_slice_size=None,
-                transposed: bool = False, accumulate: bool = True) -> None:
+                transposed: bool = False, accumulate: bool = True, tiles: Optional[TilePlan] = None) -> None:
     """lorax_sgmv_expand with an optional column window of y.  `transposed`: w_ptr addresses [L, h_out, r]
-    stacks (B^T) instead of the reference's [L, r, h_out].  accumulate=False overwrites the segments' rows."""
+    stacks (B^T) instead of the reference's [L, r, h_out].  accumulate=False overwrites the segments' rows.
+    `tiles`: a row-tile plan of the segment tables (transposed stacks only: lorax_sgmv_expand_planned)."""
     _check_sgmv(y, x, w_ptr, s_start, s_end, tmp)
     h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
+    if tiles is not None and transposed:
+        plan = tiles.c_struct(x.device)
+        with torch.cuda.device(x.device):
+            rc = lib().lorax_sgmv_expand_planned(
+                y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0),
+                x.size(0), x.size(1), h_out, int(y_offset), y.size(1), int(layer_idx), 1 if accumulate else 0,
+                ctypes.byref(plan), _dtype_code(x), _stream(x),
+            )
+        if rc != 0:
+            _raise_last(rc)
+        return
     with torch.cuda.device(x.device):
         rc = lib().lorax_sgmv_expand(
             y.data_ptr(), x.data_ptr(), w_ptr.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0),
@@ -445,10 +502,11 @@ MAX_SGMV_SHRINK_PROBLEMS = 4
 
 
 def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: float = 1.0,
-                      accumulate: bool = True) -> None:
+                      accumulate: bool = True, tiles: Optional[TilePlan] = None) -> None:
     """lorax_sgmv_shrink_multi: sgmv_shrink for up to 4 projections (outputs `ys`, pointer tables `w_ptrs`) that
     share x, the segment tables and the rank; one launch that reads x once where the kernels allow it.
-    accumulate=False overwrites the rows of the segments (no zero-fill of the outputs needed)."""
+    accumulate=False overwrites the rows of the segments (no zero-fill of the outputs needed).
+    `tiles`: a row-tile plan of the segment tables (plan_tiles, or the batch tables' own)."""
     if not 1 <= len(ys) <= MAX_SGMV_SHRINK_PROBLEMS or len(ys) != len(w_ptrs):
         raise RuntimeError(f"between 1 and {MAX_SGMV_SHRINK_PROBLEMS} outputs with one pointer table each")
     if isinstance(tmp, torch.Tensor) and tmp.dtype != torch.uint8:
@@ -461,14 +519,45 @@ def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: floa
         arr[i] = SgmvShrinkProblem(y.data_ptr(), w_ptr.data_ptr())
     if not torch.cuda.is_current_stream_capturing():
         init(x.device)
+    plan = tiles.c_struct(x.device) if tiles is not None else None
     with torch.cuda.device(x.device):
         rc = lib().lorax_sgmv_shrink_multi(
             arr, len(ys), x.data_ptr(), s_start.data_ptr(), s_end.data_ptr(), s_start.size(0), x.size(0), x.size(1),
             ys[0].size(1), int(layer_idx), float(scale), 1 if accumulate else 0, tmp.data_ptr(),
-            tmp.numel() * tmp.element_size(), _dtype_code(x), _stream(x),
+            tmp.numel() * tmp.element_size(), ctypes.byref(plan) if plan is not None else None, _dtype_code(x),
+            _stream(x),
         )
     if rc != 0:
         _raise_last(rc)
+
+
+def plan_tiles(s_start, s_end, num_tokens: int, kind: int):
+    """lorax_sgmv_plan_tiles on host copies of the segment tables (sequences of int): returns (records as a numpy
+    int32 [num_tiles, 4] array, tile_rows)."""
+    import numpy as np
+
+    starts = np.ascontiguousarray(s_start, dtype=np.int32)
+    ends = np.ascontiguousarray(s_end, dtype=np.int32)
+    if starts.shape != ends.shape or starts.ndim != 1:
+        raise RuntimeError("s_start and s_end must be one-dimensional and of one length")
+    n, rows = _c.c_int32(0), _c.c_int32(0)
+    capacity = max(16, int(num_tokens) // 16 + 2 * starts.shape[0])
+    while True:
+        records = np.empty((capacity, 4), dtype=np.int32)
+        rc = lib().lorax_sgmv_plan_tiles(starts.ctypes.data, ends.ctypes.data, starts.shape[0], int(num_tokens),
+                                         int(kind), records.ctypes.data, capacity, ctypes.byref(n), ctypes.byref(rows))
+        if rc == ESPACE:
+            capacity = int(n.value)
+            continue
+        if rc != 0:
+            raise RuntimeError(f"lorax_sgmv_plan_tiles failed with code {rc}")
+        return records[: n.value], int(rows.value)
+
+
+def set_fixed_order_shrink(on: bool) -> bool:
+    """lorax_set_fixed_order_shrink: the SGMV shrinks add their sums over the hidden dimension in one fixed order
+    whatever the batch (slower on some shapes).  Returns the previous setting."""
+    return bool(lib().lorax_set_fixed_order_shrink(1 if on else 0))
 
 
 SGMV_LORA_MAX_TOKENS = 512
@@ -515,7 +604,6 @@ def sgmv_lora_multi(problems, x, s_start, s_end, rank, layer_idx, scale: float =
         _raise_last(rc)
 
 
-ESPACE = 5
 ENTRY_DTYPE = [("adapter", "<i8"), ("a_addr", "<i8"), ("b_addr", "<i8"), ("rank", "<i4"), ("reserved", "<i4")]
 
 

@@ -192,7 +192,8 @@ class RankSegments:
                  segment_ends: Optional[torch.Tensor], indices: Optional[torch.Tensor],
                  plan: Optional[torch.Tensor] = None, lora_a_t_ptr: Optional[torch.Tensor] = None,
                  lora_b_t_ptr: Optional[torch.Tensor] = None, segments_key=None,
-                 num_long_segments: Optional[int] = None, short_plan: Optional[torch.Tensor] = None):
+                 num_long_segments: Optional[int] = None, short_plan: Optional[torch.Tensor] = None,
+                 shrink_tiles=None, expand_tiles=None):
         self.rank = rank
         self._lora_a_ptr = lora_a_ptr  # a tensor, or a function that builds it
         self._lora_b_ptr = lora_b_ptr
@@ -220,6 +221,11 @@ class RankSegments:
         # kernels over short_plan; the tables as a whole stay complete.  None / the table's length: no such plan.
         self.short_plan = short_plan
         self.num_long_segments = num_long_segments
+        # prefill: row-tile plans (_native.TilePlan) of the first num_long_segments segments for the shrink and
+        # the expand kernels, cut on the host from the segment lengths; None = the kernels search their tiles on
+        # the device
+        self.shrink_tiles = shrink_tiles
+        self.expand_tiles = expand_tiles
 
     @property
     def lora_a_ptr(self) -> Optional[torch.Tensor]:
@@ -302,6 +308,21 @@ def _segment_order(segs: List[int], seg_adapters: List[int], bounds: List[int], 
         rows[seg_adapters[s]] += bounds[s + 1] - bounds[s]
     return lambda s: (split and bounds[s + 1] - bounds[s] <= SHORT_SEGMENT_ROWS, -rows[seg_adapters[s]],
                       seg_adapters[s])
+
+
+def _tile_plans(starts: List[int], ends: List[int], num_long: int, device):
+    """Row-tile plans (shrink, expand) of the first num_long segments, cut by the library's host routine and
+    uploaded; (None, None) where the library is not loaded or the tables live on the CPU."""
+    from lorax_amd import _native
+
+    if not _native.available() or torch.device(device).type != "cuda":
+        return None, None
+    rows = max(ends[:num_long], default=0)
+    plans = []
+    for kind in (_native.TILES_SHRINK, _native.TILES_EXPAND):
+        records, tile_rows = _native.plan_tiles(starts[:num_long], ends[:num_long], rows, kind)
+        plans.append(_native.TilePlan(torch.from_numpy(records.copy()).to(device), tile_rows))
+    return plans[0], plans[1]
 
 
 class _LayoutView(Mapping):
@@ -449,7 +470,7 @@ class BatchLoraWeights(BatchAdapterWeights):
                     num_long = len(segs) - n_short
                     records = build_short_plan(segs[num_long:], seg_bounds, group_a, group_b, seg_adapters)
                     short_plan = torch.tensor(records, dtype=torch.int64, device=device).reshape(-1, BGMV_PLAN_WORDS)
-            tmp_shrink = tmp_expand = starts = ends = token_slots = plan = None
+            tmp_shrink = tmp_expand = starts = ends = token_slots = plan = shrink_tiles = expand_tiles = None
             if use_sgmv:
                 tmp_shrink, tmp_expand = get_tmp_tensors(len(segs), rank, device)
                 starts = meta.adapter_segments[segs]
@@ -458,6 +479,10 @@ class BatchLoraWeights(BatchAdapterWeights):
                     for i, s in enumerate(segs):
                         starts[i] = head_starts[s]
                         ends[i] = head_ends[s]
+                shrink_tiles, expand_tiles = _tile_plans(
+                    [head_starts[s] if head_starts is not None else seg_bounds[s] for s in segs],
+                    [head_ends[s] if head_starts is not None else seg_bounds[s + 1] for s in segs],
+                    num_long if num_long is not None else len(segs), device)
             else:
                 # slot of an adapter = position of its first segment inside this group's pointer slice
                 slot: Dict[int, int] = {}
@@ -491,6 +516,8 @@ class BatchLoraWeights(BatchAdapterWeights):
                 segments_key=(tuple(segs), head_starts is not None, chunk) if use_sgmv else None,
                 num_long_segments=num_long if num_long is not None else (len(segs) if use_sgmv else None),
                 short_plan=short_plan,
+                shrink_tiles=shrink_tiles,
+                expand_tiles=expand_tiles,
             )
 
         return cls(
@@ -750,6 +777,12 @@ def _native_batch_tables(meta: AdapterBatchMetadata, weights: Dict[str, LayerAda
                     num_long_segments=g.num_long_segments,
                     short_plan=dev64[g.plan_off // 8 : g.plan_off // 8 + g.num_chunks * BGMV_PLAN_WORDS].view(
                         g.num_chunks, BGMV_PLAN_WORDS) if g.plan_off >= 0 else None,
+                    shrink_tiles=_native.TilePlan(
+                        dev32[g.shrink_tiles_off // 4 : g.shrink_tiles_off // 4 + 4 * g.num_shrink_tiles].view(-1, 4),
+                        g.shrink_tile_rows) if g.shrink_tiles_off >= 0 else None,
+                    expand_tiles=_native.TilePlan(
+                        dev32[g.expand_tiles_off // 4 : g.expand_tiles_off // 4 + 4 * g.num_expand_tiles].view(-1, 4),
+                        g.expand_tile_rows) if g.expand_tiles_off >= 0 else None,
                 )
             else:
                 rank_data[g.rank] = RankSegments(

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "kernels.h"
+#include "sgmv_tile_plan.h"
 
 namespace {
 
@@ -81,6 +82,8 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
   std::vector<int32_t> token_seg(num_tokens);
   std::vector<int32_t> slot_count, slot_begin, slot_fill, slot_order, toks_by_slot(num_tokens), entry_first;
   std::vector<int64_t> entry_rows;
+  std::vector<int32_t> tile_starts, tile_ends;
+  std::vector<lorax_sgmv_tile_t> tile_buf;
   for (int32_t s = 0; s < num_segments; ++s)
     for (int32_t t = segment_bounds[s]; t < segment_bounds[s + 1]; ++t) token_seg[t] = s;
 
@@ -159,6 +162,7 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
         }
       }
       desc.starts_off = desc.ends_off = desc.indices_off = desc.plan_off = -1;
+      desc.shrink_tiles_off = desc.expand_tiles_off = -1;
       desc.num_long_segments = n;
       if (use_sgmv) {
         desc.starts_off = pack.reserve(static_cast<int64_t>(n) * 4);
@@ -208,6 +212,30 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
               i = j;
             }
           }
+        }
+        // Row-tile plans of the segments the segment kernels take (the long ones, when the short ones have a
+        // routing plan): the lengths are at hand, so no workgroup has to search the tables.
+        {
+          tile_starts.resize(desc.num_long_segments);
+          tile_ends.resize(desc.num_long_segments);
+          for (int32_t i = 0; i < desc.num_long_segments; ++i) {
+            tile_starts[i] = segment_bounds[segs[i]];
+            tile_ends[i] = segment_bounds[segs[i] + 1];
+          }
+          const std::vector<lorax::SegmentSpan> live =
+              lorax::live_segments(tile_starts.data(), tile_ends.data(), desc.num_long_segments, num_tokens);
+          tile_buf.clear();
+          desc.shrink_tile_rows = lorax::plan_shrink_tiles(live, tile_buf);
+          desc.num_shrink_tiles = static_cast<int32_t>(tile_buf.size());
+          desc.shrink_tiles_off = pack.reserve(static_cast<int64_t>(tile_buf.size()) * sizeof(lorax_sgmv_tile_t));
+          if (lorax_sgmv_tile_t* out = pack.at<lorax_sgmv_tile_t>(desc.shrink_tiles_off))
+            std::copy(tile_buf.begin(), tile_buf.end(), out);
+          tile_buf.clear();
+          desc.expand_tile_rows = lorax::plan_expand_tiles(live, tile_buf);
+          desc.num_expand_tiles = static_cast<int32_t>(tile_buf.size());
+          desc.expand_tiles_off = pack.reserve(static_cast<int64_t>(tile_buf.size()) * sizeof(lorax_sgmv_tile_t));
+          if (lorax_sgmv_tile_t* out = pack.at<lorax_sgmv_tile_t>(desc.expand_tiles_off))
+            std::copy(tile_buf.begin(), tile_buf.end(), out);
         }
       } else {
         // slot of a token = position of the FIRST segment of its adapter inside this group's pointer slice
@@ -268,5 +296,21 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
   *num_groups_out = num_groups;
   if (pack.used > pack.capacity || num_groups > group_capacity || (groups == nullptr && num_groups > 0))
     return LORAX_ESPACE;
+  return LORAX_OK;
+}
+
+extern "C" int lorax_sgmv_plan_tiles(const int32_t* s_start, const int32_t* s_end, int32_t num_segments,
+                                     int64_t num_tokens, int32_t kind, lorax_sgmv_tile_t* tiles, int32_t capacity,
+                                     int32_t* num_tiles, int32_t* tile_rows) {
+  if (num_segments < 0 || num_tokens < 0 || num_tiles == nullptr || tile_rows == nullptr ||
+      (num_segments > 0 && (s_start == nullptr || s_end == nullptr)) ||
+      (kind != LORAX_TILES_SHRINK && kind != LORAX_TILES_EXPAND))
+    return LORAX_EINVAL;
+  const std::vector<lorax::SegmentSpan> live = lorax::live_segments(s_start, s_end, num_segments, num_tokens);
+  std::vector<lorax_sgmv_tile_t> out;
+  *tile_rows = kind == LORAX_TILES_SHRINK ? lorax::plan_shrink_tiles(live, out) : lorax::plan_expand_tiles(live, out);
+  *num_tiles = static_cast<int32_t>(out.size());
+  if (tiles == nullptr || static_cast<size_t>(capacity < 0 ? 0 : capacity) < out.size()) return out.empty() ? LORAX_OK : LORAX_ESPACE;
+  std::copy(out.begin(), out.end(), tiles);
   return LORAX_OK;
 }

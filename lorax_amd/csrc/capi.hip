@@ -23,6 +23,7 @@ static __device__ __align__(256) unsigned char scratch[kShrinkScratchBytes];
 std::atomic<unsigned char*> g_scratch_ptr[kMaxDevices];
 
 thread_local char g_error[512] = "";
+std::atomic<int> g_fixed_order_shrink{0};
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -90,6 +91,8 @@ const Tuning& tuning() {
 #endif
   return t;
 }
+
+bool fixed_order_shrink() { return g_fixed_order_shrink.load(std::memory_order_relaxed) != 0; }
 
 }  // namespace lorax
 
@@ -168,14 +171,27 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
   return LORAX_OK;
 }
 
+// Copies a caller's row-tile plan into the launch arguments (null = the kernels search their tiles themselves).
+int take_tiles(const lorax_sgmv_tiles_t* tiles, SgmvArgs& a) {
+  if (tiles == nullptr || tiles->tiles == nullptr) return LORAX_OK;
+  if (tiles->num_tiles < 0 || tiles->tile_rows < 1 || !aligned16(tiles->tiles))
+    return fail(LORAX_EINVAL, "tile plan: num_tiles=%d tile_rows=%d tiles=%p (16-byte aligned records, tile_rows >= 1)",
+                tiles->num_tiles, tiles->tile_rows, (const void*)tiles->tiles);
+  a.tiles = reinterpret_cast<const int32_t*>(tiles->tiles);
+  a.num_tiles = tiles->num_tiles;
+  a.tile_rows = tiles->tile_rows;
+  return LORAX_OK;
+}
+
 // Shape checks and launch shared by lorax_sgmv_shrink and lorax_sgmv_shrink_static.  `scratch_buf` is
 // kShrinkScratchBytes of device memory (partial tiles, then arrival counters) or null.  A launch splits the hidden
 // dimension across workgroups only as far as the scratch has room for (sgmv_shrink_ksplit, the K parts of the
-// LDS-staged kernel), so no batch is too large for it.
+// LDS-staged kernel).  With `whole_split` a call whose split would have to be cut back for lack of room is refused
+// instead of being run with the shallower split.
 int sgmv_shrink_checked(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start, const int32_t* s_end,
                         int32_t num_segments, int64_t num_tokens, int32_t h_in, int32_t r, int32_t a_layout,
-                        int64_t layer_idx, float scale, int32_t accumulate, void* scratch_buf, int32_t dtype,
-                        void* stream) {
+                        int64_t layer_idx, float scale, int32_t accumulate, void* scratch_buf, bool whole_split,
+                        int32_t dtype, void* stream) {
   if (accumulate != 0 && accumulate != 1)
     return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (int rc = check_common(v, x, w_ptrs, dtype)) return rc;
@@ -211,8 +227,67 @@ int sgmv_shrink_checked(void* v, const void* x, const int64_t* w_ptrs, const int
   const ShrinkRoute route = sgmv_shrink_route(a);
   if (route == ShrinkRoute::kNone)
     return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d layout=%d", dtype, h_in, r, a_layout);
+  if (whole_split && (route == ShrinkRoute::kLds || route == ShrinkRoute::kRegisters)) {
+    SgmvArgs roomy = a;
+    roomy.partial_bytes = SIZE_MAX / 2;
+    const int want = route == ShrinkRoute::kLds ? sgmv_shrink_lds_kparts(a, SIZE_MAX / 2) : sgmv_shrink_ksplit(roomy);
+    const int get = route == ShrinkRoute::kLds ? sgmv_shrink_lds_kparts(a, kPartialBytes) : sgmv_shrink_ksplit(a);
+    if (want != get)
+      return fail(LORAX_ESPACE,
+                  "batch too large for the static scratch: %d parts of num_tokens * r * 4 = %lld bytes each, limit %zu "
+                  "(num_tokens=%lld r=%d); call lorax_sgmv_shrink with a tmp buffer instead",
+                  want, (long long)(num_tokens * r * 4), kPartialBytes, (long long)num_tokens, r);
+  }
   const hipError_t e = launch_sgmv_shrink(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_shrink launch failed: %s", hipGetErrorString(e));
+  return LORAX_OK;
+}
+
+// Shape checks and launch shared by lorax_sgmv_expand and lorax_sgmv_expand_planned.
+int sgmv_expand_checked(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start, const int32_t* s_end,
+                        int32_t num_segments, int64_t num_tokens, int32_t r, int32_t h_out, int32_t b_layout,
+                        int64_t y_offset, int64_t y_stride, int64_t layer_idx, int32_t accumulate,
+                        const lorax_sgmv_tiles_t* tiles, int32_t dtype, void* stream) {
+  if (accumulate != 0 && accumulate != 1)
+    return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
+  if (b_layout != LORAX_B_RH && b_layout != LORAX_B_HR) return fail(LORAX_EINVAL, "b_layout=%d", b_layout);
+  if (num_segments < 0 || num_tokens < 0)
+    return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments,
+                (long long)num_tokens);
+  if (num_segments == 0 || num_tokens == 0) return LORAX_OK;
+  if (int rc = check_common(y, v, w_ptrs, dtype)) return rc;
+  if (s_start == nullptr || s_end == nullptr)
+    return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p)", s_start, s_end);
+  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
+  if (r < 8 || r > kMaxRank || r % 8 != 0 || h_out <= 0 || h_out % 8 != 0 ||
+      num_tokens > INT32_MAX / 2)
+    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d", dtype, r, h_out);
+  if (y_offset < 0 || y_offset % 8 != 0 || y_stride % 8 != 0 || y_stride < y_offset + h_out)
+    return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld must be multiples of 8 holding h_out=%d columns",
+                (long long)y_offset, (long long)y_stride, h_out);
+  if (y_stride >= (1ll << 24))
+    return fail(LORAX_EINVAL, "y_stride=%lld: rows of y hold fewer than 2^24 elements", (long long)y_stride);
+  SgmvArgs a{};
+  a.y = y;
+  a.x = v;
+  a.w_ptrs = w_ptrs;
+  a.s_start = s_start;
+  a.s_end = s_end;
+  a.num_segments = num_segments;
+  a.num_tokens = num_tokens;
+  a.d_in = r;
+  a.d_out = h_out;
+  a.y_offset = y_offset;
+  a.y_stride = y_stride;
+  a.layer_idx = layer_idx;
+  a.dtype = dtype;
+  a.a_layout = b_layout;
+  a.accumulate = accumulate;
+  if (int rc = take_tiles(tiles, a)) return rc;
+  if (a.tiles != nullptr && a.num_tiles == 0) return LORAX_OK;  // a plan without tiles: no segment has rows
+  const hipError_t e = b_layout == LORAX_B_HR ? launch_sgmv_expand_t(a, static_cast<hipStream_t>(stream))
+                                              : launch_sgmv_expand(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_expand launch failed: %s", hipGetErrorString(e));
   return LORAX_OK;
 }
 
@@ -260,7 +335,7 @@ int lorax_sgmv_shrink(void* v, const void* x, const int64_t* w_ptrs, const int32
   // and its barrier words from tmp).  Its contents are never assumed: the counters are cleared by the launch.
   void* scratch_buf = (a_layout == LORAX_A_RH && aligned16(tmp)) ? tmp : nullptr;
   return sgmv_shrink_checked(v, x, w_ptrs, s_start, s_end, num_segments, num_tokens, h_in, r, a_layout, layer_idx,
-                             scale, 1, scratch_buf, dtype, stream);
+                             scale, 1, scratch_buf, false, dtype, stream);
 }
 
 int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, const int32_t* s_start,
@@ -279,13 +354,14 @@ int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, cons
   unsigned char* buf = nullptr;
   if (int rc = resolve_scratch(device, &buf)) return rc;
   return sgmv_shrink_checked(v, x, w_ptrs, s_start, s_end, num_segments, num_tokens, h_in, r, a_layout, layer_idx,
-                             scale, 1, buf, dtype, stream);
+                             scale, 1, buf, true, dtype, stream);
 }
 
 int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t num_problems, const void* x,
                             const int32_t* s_start, const int32_t* s_end, int32_t num_segments,
                             int64_t num_tokens, int32_t h_in, int32_t r, int64_t layer_idx, float scale,
-                            int32_t accumulate, void* tmp, int64_t tmp_bytes, int32_t dtype, void* stream) {
+                            int32_t accumulate, void* tmp, int64_t tmp_bytes, const lorax_sgmv_tiles_t* tiles,
+                            int32_t dtype, void* stream) {
   if (accumulate != 0 && accumulate != 1)
     return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
   if (num_problems < 1 || num_problems > kMaxShrinkGroup)
@@ -307,7 +383,7 @@ int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t
       if (tmp == nullptr) return fail(LORAX_EINVAL, "null pointer argument (tmp)");
       const int rc = sgmv_shrink_checked(problems[i].v, x, problems[i].w_ptrs, s_start, s_end, num_segments, num_tokens,
                                          h_in, r, LORAX_A_RH, layer_idx, scale, accumulate, aligned16(tmp) ? tmp : nullptr,
-                                         dtype, stream);
+                                         false, dtype, stream);
       if (rc != LORAX_OK) return rc;
     }
     return LORAX_OK;
@@ -350,6 +426,8 @@ int lorax_sgmv_shrink_multi(const lorax_sgmv_shrink_problem_t* problems, int32_t
     a.group.v[i] = problems[i].v;
     a.group.w[i] = problems[i].w_ptrs;
   }
+  if (int rc = take_tiles(tiles, a)) return rc;
+  if (a.tiles != nullptr && a.num_tiles == 0) return LORAX_OK;  // a plan without tiles: no segment has rows
   const hipError_t e = launch_sgmv_shrink_lds(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_shrink launch failed: %s", hipGetErrorString(e));
   return LORAX_OK;
@@ -360,48 +438,21 @@ int lorax_sgmv_expand(void* y, const void* v, const int64_t* w_ptrs, const int32
                       int32_t h_out, int32_t b_layout, int64_t y_offset, int64_t y_stride,
                       int64_t layer_idx, int32_t accumulate, void* tmp, int64_t tmp_bytes, int32_t dtype,
                       void* stream) {
-  if (accumulate != 0 && accumulate != 1)
-    return fail(LORAX_EINVAL, "accumulate=%d (0 = overwrite, 1 = add)", accumulate);
-  if (b_layout != LORAX_B_RH && b_layout != LORAX_B_HR) return fail(LORAX_EINVAL, "b_layout=%d", b_layout);
-  if (num_segments < 0 || num_tokens < 0)
-    return fail(LORAX_EINVAL, "negative size (num_segments=%d num_tokens=%lld)", num_segments,
-                (long long)num_tokens);
-  if (tmp_bytes != static_cast<int64_t>(lorax_sgmv_tmp_size(num_segments)))  // punica_ops.cc:359
+  if (num_segments >= 0 && tmp_bytes != static_cast<int64_t>(lorax_sgmv_tmp_size(num_segments)))  // punica_ops.cc:359
     return fail(LORAX_ETMPSIZE, "CHECK_EQ(tmp.size(0), sgmv_tmp_size(num_problems)) failed. %lld vs %zu",
                 (long long)tmp_bytes, lorax_sgmv_tmp_size(num_segments));
-  if (num_segments == 0 || num_tokens == 0) return LORAX_OK;
-  if (int rc = check_common(y, v, w_ptrs, dtype)) return rc;
-  if (s_start == nullptr || s_end == nullptr || (tmp == nullptr && tmp_bytes > 0))
-    return fail(LORAX_EINVAL, "null pointer argument (s_start=%p s_end=%p tmp=%p)", s_start, s_end, tmp);
-  if (layer_idx < 0) return fail(LORAX_EINVAL, "layer_idx=%lld is negative", (long long)layer_idx);
-  if (r < 8 || r > kMaxRank || r % 8 != 0 || h_out <= 0 || h_out % 8 != 0 ||
-      num_tokens > INT32_MAX / 2)
-    return fail(LORAX_ENOKERNEL, "No suitable kernel. dtype=%d d_in=%d d_out=%d", dtype, r, h_out);
-  if (y_offset < 0 || y_offset % 8 != 0 || y_stride % 8 != 0 || y_stride < y_offset + h_out)
-    return fail(LORAX_EINVAL, "y_offset=%lld y_stride=%lld must be multiples of 8 holding h_out=%d columns",
-                (long long)y_offset, (long long)y_stride, h_out);
-  if (y_stride >= (1ll << 24))
-    return fail(LORAX_EINVAL, "y_stride=%lld: rows of y hold fewer than 2^24 elements", (long long)y_stride);
-  SgmvArgs a{};
-  a.y = y;
-  a.x = v;
-  a.w_ptrs = w_ptrs;
-  a.s_start = s_start;
-  a.s_end = s_end;
-  a.num_segments = num_segments;
-  a.num_tokens = num_tokens;
-  a.d_in = r;
-  a.d_out = h_out;
-  a.y_offset = y_offset;
-  a.y_stride = y_stride;
-  a.layer_idx = layer_idx;
-  a.dtype = dtype;
-  a.a_layout = b_layout;
-  a.accumulate = accumulate;
-  const hipError_t e = b_layout == LORAX_B_HR ? launch_sgmv_expand_t(a, static_cast<hipStream_t>(stream))
-                                              : launch_sgmv_expand(a, static_cast<hipStream_t>(stream));
-  if (e != hipSuccess) return fail(LORAX_ELAUNCH, "sgmv_expand launch failed: %s", hipGetErrorString(e));
-  return LORAX_OK;
+  if (num_segments > 0 && num_tokens > 0 && tmp == nullptr && tmp_bytes > 0)
+    return fail(LORAX_EINVAL, "null pointer argument (tmp)");
+  return sgmv_expand_checked(y, v, w_ptrs, s_start, s_end, num_segments, num_tokens, r, h_out, b_layout, y_offset,
+                             y_stride, layer_idx, accumulate, nullptr, dtype, stream);
+}
+
+int lorax_sgmv_expand_planned(void* y, const void* v, const int64_t* w_ptrs, const int32_t* s_start,
+                              const int32_t* s_end, int32_t num_segments, int64_t num_tokens, int32_t r,
+                              int32_t h_out, int64_t y_offset, int64_t y_stride, int64_t layer_idx,
+                              int32_t accumulate, const lorax_sgmv_tiles_t* tiles, int32_t dtype, void* stream) {
+  return sgmv_expand_checked(y, v, w_ptrs, s_start, s_end, num_segments, num_tokens, r, h_out, LORAX_B_HR, y_offset,
+                             y_stride, layer_idx, accumulate, tiles, dtype, stream);
 }
 
 int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems, int64_t num_tokens,
@@ -510,6 +561,8 @@ int lorax_init(int32_t device) {
   if (e != hipSuccess) return fail(LORAX_ELAUNCH, "kernel set-up on device %d: %s", device, hipGetErrorString(e));
   return LORAX_OK;
 }
+
+int lorax_set_fixed_order_shrink(int32_t on) { return g_fixed_order_shrink.exchange(on != 0 ? 1 : 0); }
 
 size_t lorax_workspace_bytes(void) { return kShrinkScratchBytes; }
 

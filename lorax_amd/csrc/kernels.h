@@ -95,6 +95,10 @@ struct SgmvArgs {
   size_t partial_bytes;
   uint32_t* counters;
   size_t num_counters;
+  // optional row-tile plan of the caller (lorax_sgmv_tiles_t): device records, their number, their height bound
+  const int32_t* tiles;
+  int num_tiles;
+  int tile_rows;
 };
 
 // Shrink and expand of a short prefill batch in one launch (bgmv.hip): up to four projections that share x and
@@ -148,6 +152,9 @@ struct Tuning {
   int bgmv_scalar_y;    // LORAX_BGMV_SCALAR_Y: BGMV expand that moves y element by element even where rows are aligned
 };
 const Tuning& tuning();
+// lorax_set_fixed_order_shrink: the SGMV shrinks walk the hidden dimension from k = 0 in every tile and never cut
+// it across workgroups.
+bool fixed_order_shrink();
 
 hipError_t launch_bgmv(const BgmvArgs& a, hipStream_t stream);
 hipError_t launch_bgmv_lora(const BgmvArgs& a, hipStream_t stream);
@@ -184,5 +191,7 @@ constexpr size_t kPartialBytes = kShrinkScratchBytes - kShrinkCounterBytes;
 constexpr size_t kNumCounters = kShrinkCounterBytes / sizeof(uint32_t);
 // K splits the register-operand shrink would use for this call given its scratch (1 = none).
 int sgmv_shrink_ksplit(const SgmvArgs& a);
+// Parts the LDS-staged shrink would cut the hidden dimension into given `room` bytes for their fp32 sums.
+int sgmv_shrink_lds_kparts(const SgmvArgs& a, size_t room);
 
 }  // namespace lorax

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     const int64_t* __restrict__ W, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int r, int h_out,
     int64_t y_offset, int64_t y_stride, int64_t layer_idx, int rows_per_tile, int panels_per_wave,
-    int tile_slots, int accumulate_into_y) {
+    int tile_slots, int accumulate_into_y, const TileList plan) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   typedef E yvec __attribute__((ext_vector_type(NJ)));
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     RowTile rt;
     // small remainders are merged into the segment's other tiles: a tile's prologue (the search and the panel
     // operands) costs as much as a hundred rows
-    if (!find_row_tile<true>(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
+    if (!get_row_tile<true>(plan, s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const E* BT = reinterpret_cast<const E*>(segment_entry(pre_w, W, rt.seg)) + layer_idx * h_out * static_cast<int64_t>(r);
     const int nmb = (rt.row_end - rt.row0 + 15) / 16;
 
@@ -181,7 +181,12 @@ static hipError_t launch_expand_t_ks(const SgmvArgs& a, hipStream_t stream) {
   // high (merged remainders): rows of more than 2^23 elements get lower tiles.
   while (rows_per_tile > 16 && a.y_stride * (rows_per_tile + rows_per_tile / 8 + 16) >= (1ll << 32)) rows_per_tile /= 2;
   if (a.y_stride * (rows_per_tile + rows_per_tile / 8 + 16) >= (1ll << 32)) return hipErrorInvalidValue;
-  const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
+  // With the caller's tile plan the tile count is exact (no workgroup without work) and a tile is at most
+  // tile_rows high; the plan is ignored when its tiles would overflow the 32-bit offsets.
+  const bool planned = a.tiles != nullptr && a.num_tiles > 0 && a.tile_rows >= 1 && tuning().expand_rows == 0 &&
+                       a.y_stride * static_cast<int64_t>(a.tile_rows) < (1ll << 32);
+  const int64_t tiles = planned ? a.num_tiles : (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
+  const TileList plan{planned ? a.tiles : nullptr, planned ? a.num_tiles : 0, planned ? a.tile_rows : 0};
   constexpr int kCols = 16 * NJ;
   const int num_panels = (a.d_out + kCols - 1) / kCols;
   // Panels per wave: more of them amortise the tile search, fewer give more workgroups; keep a few
@@ -195,7 +200,7 @@ static hipError_t launch_expand_t_ks(const SgmvArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((sgmv_expand_t_kernel<D, KS, NJ>), grid, dim3(kExpTThreads), 0, stream,
                      static_cast<typename D::E*>(a.y), static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start,
                      a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.d_out, a.y_offset,
-                     a.y_stride, a.layer_idx, rows_per_tile, ppw, tile_slots, a.accumulate);
+                     a.y_stride, a.layer_idx, rows_per_tile, ppw, tile_slots, a.accumulate, plan);
   return hipGetLastError();
 }
 

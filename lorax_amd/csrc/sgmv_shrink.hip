@@ -291,6 +291,7 @@ int sgmv_shrink_ksplit(const SgmvArgs& a) {
   const int64_t tiles = (a.num_tokens + mb * 16 - 1) / (mb * 16) + a.num_segments;
   const int ksteps = (a.d_in + 31) / 32;
   int ksplit = 1;
+  if (fixed_order_shrink()) return 1;
   if (tuning().shrink_ksplit > 0) {
     ksplit = tuning().shrink_ksplit;
   } else if (tiles < 192) {
@@ -323,7 +324,8 @@ static hipError_t launch_rh_w(const SgmvArgs& a, int ksplit, hipStream_t stream)
                      stream, static_cast<typename D::E*>(a.y),
                      static_cast<const typename D::E*>(a.x), a.w_ptrs, a.s_start, a.s_end,
                      a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, ksplit,
-                     a.partials, a.counters, static_cast<int>(a.num_counters), tuning().shrink_no_rotate ? 0 : 1, a.scale,
+                     a.partials, a.counters, static_cast<int>(a.num_counters),
+                     (tuning().shrink_no_rotate || fixed_order_shrink()) ? 0 : 1, a.scale,
                      a.accumulate);
   return hipGetLastError();
 }

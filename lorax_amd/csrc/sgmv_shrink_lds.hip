@@ -61,7 +61,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     const ShrinkGroup grp, const typename D::E* __restrict__ X, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int h_in, int64_t layer_idx,
     int stages, float scale, int accumulate_into_v, int rows_per_tile, int kparts, int tile_slots,
-    float* __restrict__ partials, int rotate) {
+    float* __restrict__ partials, int rotate, const TileList plan) {
   using E = typename D::E;
   using vec8 = typename D::vec8;
   // The A tile stacks the A matrices of grp.count projections of rank r: row p * r + i is row i of
@@ -108,15 +108,24 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
   const int nst = static_cast<int>(static_cast<int64_t>(kpart + 1) * (h_in / kLdsKc) / kparts) - st_begin;
   const int k_begin = st_begin * kLdsKc;
 
+  // the projections' table entries of the first 64 segments travel with the tile's own loads (sgmv_tiles.h)
+  int64_t pre_w[kMaxShrinkGroup];
+#pragma unroll
+  for (int p = 0; p < kMaxShrinkGroup; ++p) pre_w[p] = preload_segment_entry(grp.w[p < grp.count ? p : 0], num_segments);
+
   for (int tile = first_tile;; tile += gridDim.x) {
     if (kparts > 1 && tile != first_tile) break;  // one tile per workgroup when K is split
     RowTile rt;
     // tiles may be lower than the ROWS the buffers hold: rows past a tile's end re-read its last row
-    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
+    if (!get_row_tile(plan, s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const E* A[kMaxShrinkGroup];
+    int64_t stack0 = 0;
 #pragma unroll
-    for (int p = 0; p < kMaxShrinkGroup; ++p)
-      A[p] = reinterpret_cast<const E*>(grp.w[p < grp.count ? p : 0][rt.seg]) + layer_idx * r * static_cast<int64_t>(h_in);
+    for (int p = 0; p < kMaxShrinkGroup; ++p) {
+      const int64_t stack = segment_entry(pre_w[p], grp.w[p < grp.count ? p : 0], rt.seg);
+      if (p == 0) stack0 = stack;
+      A[p] = reinterpret_cast<const E*>(stack) + layer_idx * r * static_cast<int64_t>(h_in);
+    }
 
     // Source addresses of this thread's chunks.  Load j of a thread covers chunk id j * 256 + tid of
     // the tile: row = id / 16, position = id % 16, and it fetches the row's chunk position ^ (row & 15).
@@ -144,7 +153,7 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     // or 56 KB where staggered walks reach 6.0-6.5 TB/s.  The tiles of one segment that run on one XCD stay
     // within a few stages of each other, so that they still find the segment's A tiles in that XCD's L2.
     // Tiles that read the same stack of A (one adapter, whatever the segment) keep the same start.
-    const unsigned who = static_cast<unsigned>(reinterpret_cast<uintptr_t>(A[0]) >> 12) * 2654435761u >> 20;
+    const unsigned who = static_cast<unsigned>(static_cast<uint64_t>(stack0) >> 12) * 2654435761u >> 20;
     const int rot = rotate ? static_cast<int>((37u * (who * kXcds + blockIdx.x % kXcds) +
                                                static_cast<unsigned>(rt.index) % 8u) % static_cast<unsigned>(nst))
                            : 0;
@@ -260,13 +269,13 @@ template <typename D>
 __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_parts_kernel(
     const ShrinkGroup grp, const float* __restrict__ partials, const int32_t* __restrict__ s_start,
     const int32_t* __restrict__ s_end, int num_segments, int num_tokens, int R, int kparts, float scale,
-    int accumulate_into_v, int rows_per_tile) {
+    int accumulate_into_v, int rows_per_tile, const TileList plan) {
   using E = typename D::E;
   const int r = grp.rank;
   const int n4 = grp.count * r / 4;  // groups of 4 adjacent columns per row (r is a multiple of 8)
   for (int tile = blockIdx.x;; tile += gridDim.x) {
     RowTile rt;
-    if (!find_row_tile(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
+    if (!get_row_tile(plan, s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const int n = (rt.row_end - rt.row0) * n4;
     for (int i = threadIdx.x; i < n; i += kLdsThreads) {
       const int row = rt.row0 + i / n4;
@@ -302,59 +311,98 @@ static hipError_t raise_lds_limit() {
   return hipSuccess;
 }
 
-template <typename D, int NB, int MBLK, bool KSPLIT>
-static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_rows = 0) {
-  constexpr int kStageBytes = (MBLK + NB) * 16 * kLdsRowBytes;
-  constexpr int kRedBytes = KSPLIT ? 4 * MBLK * NB * 1024 : 0;  // partial sums of the four waves at the end of a tile
-  static_assert(kRedBytes <= kLdsMaxBytes, "partial sums must fit in LDS");
-  // Tile height: a launch streams at the rate of the CUs that have a workgroup, so when the full-height tiles
-  // are fewer than the 256 CUs the tiles are lowered (in steps of 16 rows) until they are about as many.  The
-  // host knows the rows and the number of segments, not their lengths: ceil(T / M) + segments bounds the count.
-  int rows_per_tile = MBLK * 16;
-  if (fixed_rows > 0) {
-    rows_per_tile = fixed_rows;
-  } else if (tuning().shrink_rows <= 0) {
-    while (rows_per_tile > 16 &&
-           (a.num_tokens + rows_per_tile - 17) / (rows_per_tile - 16) + a.num_segments <= 256)
-      rows_per_tile -= 16;
-  } else if (tuning().shrink_rows < rows_per_tile) {
-    rows_per_tile = (tuning().shrink_rows + 15) / 16 * 16;
-  }
-  // Tiles of 48 rows in buffers of 48: the fourth row block of 64-row buffers would be staged (re-reading the
-  // tile's last row) and multiplied for nothing.  With three row blocks the waves take k slices at every rank
-  // (96 accumulator registers per lane at rank 128; cfg3's stacked gate/up launch 37.0 -> 34.8 us against the
-  // waves splitting the output blocks).
-  if constexpr (MBLK == 4) {
-    constexpr bool kSlices = KSPLIT || NB > 4;
-    if constexpr (kSlices || NB % 4 == 0) {  // (output blocks of three row blocks only divide as 1 x 4)
-      if (rows_per_tile == 48 && fixed_rows == 0 && tuning().shrink_mb == 0)
-        return launch_lds_m<D, NB, 3, kSlices>(a, stream, 48);
+// What a launch looks like: decided from host-known sizes only (and from the caller's tile plan, which knows the
+// tiles exactly), so that the same call always runs the same way.
+struct LdsLaunch {
+  int mblk;           // 16-row blocks of the stage buffers (1, 2, 3, 4)
+  bool kslices;       // the four waves split the k slices of a stage (else the output blocks)
+  int rows_per_tile;  // tile height, at most 16 * mblk
+  int64_t tiles;      // row tiles: exact with a plan, else an upper bound
+  bool planned;
+  int kparts;         // parts the hidden dimension is cut into across workgroups (1 = none)
+};
+
+// `room`: bytes of scratch for the K parts' fp32 sums.
+static LdsLaunch lds_launch_shape(const SgmvArgs& a, size_t room) {
+  const int NB = (a.d_out + 15) / 16;
+  LdsLaunch l{};
+  const bool kslices_pref = tuning().shrink_lds != 2;
+  l.planned = a.tiles != nullptr && a.num_tiles > 0 && a.tile_rows >= 1 && a.tile_rows <= 64 && tuning().shrink_mb == 0 &&
+              tuning().shrink_rows == 0;
+  if (l.planned) {
+    // the plan's tiles in buffers just high enough; the waves take k slices wherever that variant exists
+    l.mblk = (a.tile_rows + 15) / 16;
+    l.rows_per_tile = l.mblk * 16;
+    l.kslices = l.mblk != 4 || NB <= 4;
+    l.tiles = a.num_tiles;
+  } else {
+    // Row-tile height: the tallest of 64 / 32 / 16 rows that still yields 128 tiles (a workgroup streams about
+    // 50 GB/s, so fewer, larger tiles leave HBM idle) and is not much taller than the average segment (rows past a
+    // segment's end are padding).  Short tiles re-read A more often, but from L2.
+    const int64_t avg_len = a.num_tokens / (a.num_segments > 0 ? a.num_segments : 1);
+    int mblk = 4;
+    while (mblk > 1 && ((a.num_tokens + mblk * 16 - 1) / (mblk * 16) + a.num_segments < 128 || mblk * 8 > avg_len))
+      mblk /= 2;
+    if (tuning().shrink_mb > 0) mblk = tuning().shrink_mb;
+    if (mblk != 1 && mblk != 2 && mblk != 4) mblk = 1;
+    // every staged byte read from LDS once (k slices per wave) up to rank 64 in 64-row buffers; above, the waves
+    // split the output blocks instead (k slices at rank 128 need 128 accumulator registers per lane and measured
+    // no faster)
+    l.mblk = mblk;
+    l.kslices = mblk == 4 ? (NB <= 4 && kslices_pref) : (mblk == 2 ? !(NB % 2 == 0 && !kslices_pref) : true);
+    // A launch streams at the rate of the CUs that have a workgroup, so when the full-height tiles are fewer than
+    // the 256 CUs the tiles are lowered (in steps of 16 rows) until they are about as many.  The host knows the
+    // rows and the number of segments, not their lengths: ceil(T / M) + segments bounds the count.
+    int rows = mblk * 16;
+    if (tuning().shrink_rows <= 0) {
+      while (rows > 16 && (a.num_tokens + rows - 17) / (rows - 16) + a.num_segments <= 256) rows -= 16;
+    } else if (tuning().shrink_rows < rows) {
+      rows = (tuning().shrink_rows + 15) / 16 * 16;
     }
+    // Tiles of 48 rows in buffers of 48: the fourth row block of 64-row buffers would be staged (re-reading the
+    // tile's last row) and multiplied for nothing.  With three row blocks the waves take k slices at every rank
+    // (96 accumulator registers per lane at rank 128; a stacked gate/up launch of rank 128 37.0 -> 34.8 us
+    // against the waves splitting the output blocks).
+    if (mblk == 4 && rows == 48 && tuning().shrink_mb == 0 && (l.kslices || NB > 4 || NB % 4 == 0)) {
+      l.mblk = 3;
+      l.kslices = l.kslices || NB > 4;
+    }
+    l.rows_per_tile = rows;
+    l.tiles = (a.num_tokens + rows - 1) / rows + a.num_segments;
   }
-  const int64_t tiles = (a.num_tokens + rows_per_tile - 1) / rows_per_tile + a.num_segments;
   // K parts: a workgroup streams its tile's x and A at about 50 GB/s whatever the launch, so a launch of a
   // hundred tiles (a prefill batch of one or two thousand rows) leaves most of the chip idle.  Its hidden
-  // dimension is cut into parts of at least 8 stages, about one workgroup per CU (two measured no faster), and a
-  // second small launch adds the parts.  Needs the scratch (fp32 sums, kparts x rows x R); decided from
-  // host-known sizes only.
-  constexpr int R = NB * 16;
-  int kparts = 1;
+  // dimension is cut into parts of at least 8 stages and a second small launch adds the parts.  Up to 120 tiles:
+  // about one workgroup per CU (two measured no faster).  Up to 192 tiles (a single long run of a few thousand
+  // rows cut into 32-row tiles): two or three parts, about two workgroups per CU - measured on a 4096-row run at
+  // rank 128, 140 tiles: 51 -> 40 us over h_in = 8192 and 145 -> 86 us over h_in = 28672 with three parts (two: 45
+  // and 116 us; four and more, which no longer fit the CUs at once: 46 and 104 us).  Launches with more tiles
+  // than that are slower with parts than without (254 tiles in two parts: 27 against 23 us).  Needs the scratch
+  // (fp32 sums, kparts x rows x R).
+  const int R = NB * 16;
   const int nst_all = a.d_in / kLdsKc;
-  // Up to 128 tiles: about one workgroup per CU.  Up to 192 tiles (a single long run of a few thousand rows cut
-  // into 32-row tiles): two or three parts, about two workgroups per CU - measured on a 4096-row run at rank 128,
-  // 140 tiles: 51 -> 40 us over h_in = 8192 and 145 -> 86 us over h_in = 28672 with three parts (two: 45 and 116 us;
-  // four and more, which no longer fit the CUs at once: 46 and 104 us).  Launches with more tiles than that are
-  // slower with parts than without (254 tiles in two parts: 27 against 23 us).
-  if (a.partials != nullptr && (tiles < 192 || tuning().shrink_ksplit > 0)) {
-    kparts = static_cast<int>((tiles <= 128 ? 256 : 512) / tiles);
+  l.kparts = 1;
+  if (a.partials != nullptr && !fixed_order_shrink() && (l.tiles < 192 || tuning().shrink_ksplit > 0)) {
+    // (121 to 170 tiles: three parts - a 4096-row run in exactly 128 tiles measured 45 us in two parts, 40 us in three)
+    const int64_t nt = l.tiles > 0 ? l.tiles : 1;
+    int kparts = static_cast<int>(nt <= 120 ? 256 / nt : (512 / nt < 3 ? 512 / nt : 3));
     if (kparts > 8) kparts = 8;
     if (kparts > nst_all / 8) kparts = nst_all / 8;
     if (tuning().shrink_ksplit > 0) kparts = tuning().shrink_ksplit < nst_all ? tuning().shrink_ksplit : nst_all;
-    // (the first 8 MiB whatever the buffer's size, so that the result does not depend on it)
-    const size_t room = a.partial_bytes < kPartialBytes ? a.partial_bytes : kPartialBytes;
     while (kparts > 1 && static_cast<size_t>(kparts) * a.num_tokens * R * sizeof(float) > room) --kparts;
-    if (kparts < 1) kparts = 1;
+    l.kparts = kparts < 1 ? 1 : kparts;
   }
+  return l;
+}
+
+template <typename D, int NB, int MBLK, bool KSPLIT>
+static hipError_t launch_lds_m(const SgmvArgs& a, const LdsLaunch& l, hipStream_t stream) {
+  constexpr int kStageBytes = (MBLK + NB) * 16 * kLdsRowBytes;
+  constexpr int kRedBytes = KSPLIT ? 4 * MBLK * NB * 1024 : 0;  // partial sums of the four waves at the end of a tile
+  static_assert(kRedBytes <= kLdsMaxBytes, "partial sums must fit in LDS");
+  constexpr int R = NB * 16;
+  const int64_t tiles = l.tiles;
+  const int kparts = l.kparts;
   const int64_t wgs = tiles * kparts;
   // Stage buffers: all of a CU's LDS when there is at most one workgroup per CU; a third of it when the
   // workgroups make one to three rounds over the CUs (more resident workgroups even out the last round);
@@ -379,44 +427,42 @@ static hipError_t launch_lds_m(const SgmvArgs& a, hipStream_t stream, int fixed_
     grp.count = 1;
     grp.rank = a.d_out;
   }
+  const TileList plan{l.planned ? a.tiles : nullptr, l.planned ? a.num_tiles : 0, l.rows_per_tile};
+  const int rotate = (tuning().shrink_no_rotate || fixed_order_shrink()) ? 0 : 1;
   hipLaunchKernelGGL(kernel, grid, dim3(kLdsThreads), lds_bytes, stream, grp, static_cast<const typename D::E*>(a.x),
                      a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), a.d_in, a.layer_idx, stages,
-                     a.scale, a.accumulate, rows_per_tile, kparts, static_cast<int>(tiles), a.partials,
-                     tuning().shrink_no_rotate ? 0 : 1);
+                     a.scale, a.accumulate, l.rows_per_tile, kparts, static_cast<int>(tiles), a.partials, rotate, plan);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess || kparts == 1) return e;
   hipLaunchKernelGGL(sgmv_shrink_parts_kernel<D>, dim3(static_cast<unsigned>(tiles)), dim3(kLdsThreads), 0, stream, grp,
                      a.partials, a.s_start, a.s_end, a.num_segments, static_cast<int>(a.num_tokens), R, kparts, a.scale,
-                     a.accumulate, rows_per_tile);
+                     a.accumulate, l.rows_per_tile, plan);
   return hipGetLastError();
 }
 
 template <typename D, int NB>
 static hipError_t launch_lds_nb(const SgmvArgs& a, hipStream_t stream) {
-  // Row-tile height: the tallest of 64 / 32 / 16 rows that still yields 128 tiles (a workgroup streams
-  // about 50 GB/s, so fewer, larger tiles leave HBM idle) and is not much taller than the average
-  // segment (rows past a segment's end are padding).  Short tiles re-read A more often, but from L2.
-  const int64_t avg_len = a.num_tokens / (a.num_segments > 0 ? a.num_segments : 1);
-  int mblk = 4;
-  while (mblk > 1 && ((a.num_tokens + mblk * 16 - 1) / (mblk * 16) + a.num_segments < 128 || mblk * 8 > avg_len))
-    mblk /= 2;
-  if (tuning().shrink_mb > 0) mblk = tuning().shrink_mb;
-  const bool ksplit = tuning().shrink_lds != 2;
-  if (mblk >= 4) {
-    // every staged byte read from LDS once (k slices per wave) up to rank 64; above, the waves split the output
-    // blocks instead (k slices at rank 128 need 128 accumulator registers per lane and measured no faster)
-    if constexpr (NB <= 4) {
-      if (ksplit) return launch_lds_m<D, NB, 4, true>(a, stream);
-    }
-    return launch_lds_m<D, NB, 4, false>(a, stream);
+  // (the first 8 MiB of the scratch whatever the buffer's size, so that the result does not depend on it)
+  const LdsLaunch l = lds_launch_shape(a, a.partial_bytes < kPartialBytes ? a.partial_bytes : kPartialBytes);
+  switch (l.mblk) {
+    case 4:
+      if constexpr (NB <= 4) {
+        if (l.kslices) return launch_lds_m<D, NB, 4, true>(a, l, stream);
+      }
+      return launch_lds_m<D, NB, 4, false>(a, l, stream);
+    case 3:
+      if constexpr (NB <= 4 && NB % 4 == 0) {
+        if (!l.kslices) return launch_lds_m<D, NB, 3, false>(a, l, stream);
+      }
+      return launch_lds_m<D, NB, 3, true>(a, l, stream);
+    case 2:
+      if constexpr (NB % 2 == 0) {
+        if (!l.kslices) return launch_lds_m<D, NB, 2, false>(a, l, stream);
+      }
+      return launch_lds_m<D, NB, 2, true>(a, l, stream);
+    default:
+      return launch_lds_m<D, NB, 1, true>(a, l, stream);
   }
-  if (mblk == 2) {
-    if constexpr (NB % 2 == 0) {
-      if (!ksplit) return launch_lds_m<D, NB, 2, false>(a, stream);
-    }
-    return launch_lds_m<D, NB, 2, true>(a, stream);
-  }
-  return launch_lds_m<D, NB, 1, true>(a, stream);
 }
 
 template <typename D>
@@ -478,6 +524,8 @@ hipError_t configure_sgmv_shrink_lds() {
   const hipError_t e = raise_lds_limits_dtype<F16>();
   return e != hipSuccess ? e : raise_lds_limits_dtype<BF16>();
 }
+
+int sgmv_shrink_lds_kparts(const SgmvArgs& a, size_t room) { return lds_launch_shape(a, room).kparts; }
 
 bool sgmv_shrink_lds_applies(const SgmvArgs& a) {
   return a.a_layout == LORAX_A_RH && a.d_in % kLdsKc == 0 && a.d_out % 8 == 0 && a.d_out >= 8 && a.d_out <= 128;

@@ -106,6 +106,30 @@ __device__ __forceinline__ bool find_row_tile(const int32_t* __restrict__ s_star
   return false;
 }
 
+// A launch's row tiles: from the caller's plan when it brought one (one 16-byte record per tile, wave-uniform
+// address: a scalar load), else by the search above.  Records are clamped to the call's sizes - a wrong plan gives
+// wrong results, but no access outside the call's tensors - and a record without rows ends the workgroup's walk.
+struct TileList {
+  const int32_t* records;  // lorax_sgmv_tile_t[num_tiles] in device memory, or null
+  int num_tiles;
+  int max_rows;            // no tile is higher
+};
+
+template <bool MERGE = false>
+__device__ __forceinline__ bool get_row_tile(const TileList& plan, const int32_t* __restrict__ s_start,
+                                             const int32_t* __restrict__ s_end, int num_segments, int num_tokens,
+                                             int rows_per_tile, int tile, RowTile& out) {
+  if (plan.records == nullptr) return find_row_tile<MERGE>(s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, out);
+  if (tile >= plan.num_tiles || num_segments <= 0) return false;
+  typedef int int32x4 __attribute__((ext_vector_type(4)));
+  const int32x4 rec = *reinterpret_cast<const int32x4*>(plan.records + 4 * static_cast<int64_t>(tile));
+  out.seg = min(max(rec[0], 0), num_segments - 1);
+  out.row0 = min(max(rec[1], 0), num_tokens);
+  out.row_end = min(min(rec[2], num_tokens), out.row0 + plan.max_rows);
+  out.index = rec[3];
+  return out.row_end > out.row0;
+}
+
 // The stack address of a tile's segment without a memory round trip after the tile search: every lane asks for
 // the table entry of "its" segment BEFORE the search (the loads travel together with the search's own), and the
 // entry of the segment the search lands on is read from that lane afterwards.  Segments past the first 64 fall

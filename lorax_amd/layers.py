@@ -123,9 +123,10 @@ class LoraLinear(nn.Module):
                     if rs.segments_key is not None and rs.lora_b_t_ptr is not None and not tensor_parallel:
                         prefill_jobs[(r, rs.segments_key)].append((rs, start, end - start))
                         continue
+                    whole = rs.num_long_segments == rs.segment_starts.numel()  # the plans cover the long segments
                     v = lora_a_sgmv_resident(
                         input, get_shrink_scratch(input.device), rs.lora_a_t_ptr, rs.segment_starts, rs.segment_ends,
-                        self.layer_id, r, zero_fill=tensor_parallel,
+                        self.layer_id, r, zero_fill=tensor_parallel, tiles=rs.shrink_tiles if whole else None,
                     )
                 else:
                     if rs.lora_a_ptr is None:
@@ -139,9 +140,10 @@ class LoraLinear(nn.Module):
                 if tensor_parallel:
                     v = self.collect_lora_a(v)
                 if rs.lora_b_t_ptr is not None:
+                    whole = rs.num_long_segments == rs.segment_starts.numel()
                     lora_b_sgmv_cutlass_slice(
                         result, v, rs.tmp_expand, rs.lora_b_t_ptr, rs.segment_starts, rs.segment_ends,
-                        self.layer_id, start, end - start, transposed=True,
+                        self.layer_id, start, end - start, transposed=True, tiles=rs.expand_tiles if whole else None,
                     )
                 elif sliced:
                     lora_b_sgmv_cutlass_slice(
@@ -179,6 +181,10 @@ class LoraLinear(nn.Module):
                      and all(p.size(0) <= _native.MAX_BGMV_TOKENS for p in plans))
             n_long = first.num_long_segments if split else first.segment_starts.numel()
             starts, ends = first.segment_starts[:n_long], first.segment_ends[:n_long]
+            # the tables' row-tile plans cover their first num_long_segments entries
+            planned = n_long == first.num_long_segments
+            shrink_tiles = first.shrink_tiles if planned else None
+            expand_tiles = first.expand_tiles if planned else None
             # v needs no zero-fill: the shrinks overwrite the rows of their segments and the expands read no others
             flat = torch.empty((len(group), input.size(0), r), dtype=input.dtype, device=input.device)
             vs = list(flat.unbind(0))
@@ -187,7 +193,7 @@ class LoraLinear(nn.Module):
             for i in range(0, len(group) if n_long > 0 else 0, step):
                 _native.sgmv_shrink_multi(
                     vs[i : i + step], input, [rs.lora_a_t_ptr[:n_long] for rs, _, _ in group[i : i + step]],
-                    starts, ends, get_shrink_scratch(input.device), self.layer_id, 1.0, False,
+                    starts, ends, get_shrink_scratch(input.device), self.layer_id, 1.0, False, shrink_tiles,
                 )
             batch = _native.MAX_BGMV_PROBLEMS
             if split:  # the short rows of every projection of the group in one launch
@@ -197,7 +203,7 @@ class LoraLinear(nn.Module):
             for v, (rs, start, width) in zip(vs, group) if n_long > 0 else ():
                 lora_b_sgmv_cutlass_slice(
                     result, v, rs.tmp_expand[: get_tmp_expand_size(n_long)], rs.lora_b_t_ptr[:n_long], starts, ends,
-                    self.layer_id, start, width, transposed=True,
+                    self.layer_id, start, width, transposed=True, tiles=expand_tiles,
                 )
             if split:
                 for i in range(0, len(group), batch):

@@ -158,6 +158,7 @@ def lora_a_sgmv_resident(
     layer_idx: int,
     lora_rank: int,
     zero_fill: bool = True,
+    tiles=None,
 ) -> torch.Tensor:
     """As lora_a_sgmv_cutlass, reading the [L, r, h_in] stacks of the decode path (weights_a_t) whatever
     the rank.  `tmp` is get_shrink_scratch(device) or the 8 MiB buffer of get_tmp_tensor.
@@ -165,7 +166,7 @@ def lora_a_sgmv_resident(
     outside every segment hold garbage - fine for a v that only goes to the expand of the same segments."""
     alloc = torch.zeros if zero_fill else torch.empty
     v = alloc((x.size(0), lora_rank), dtype=x.dtype, device=x.device)
-    _native_module().sgmv_shrink_multi([v], x, [wa_t_ptr], s_start, s_end, tmp, layer_idx, 1.0, zero_fill)
+    _native_module().sgmv_shrink_multi([v], x, [wa_t_ptr], s_start, s_end, tmp, layer_idx, 1.0, zero_fill, tiles)
     return v
 
 
@@ -262,11 +263,12 @@ def add_lora_b_bgmv_slice(y, v, wb_T_all, indicies, layer_idx, y_offset: int, y_
 
 
 def lora_b_sgmv_cutlass_slice(y, v, tmp, wb_ptr, s_start, s_end, layer_idx, y_offset: int, y_slice_size: int,
-                              transposed: bool = False):
+                              transposed: bool = False, tiles=None):
     """As lora_b_sgmv_cutlass, writing columns [y_offset, y_offset + y_slice_size) of a wider y.  With
     `transposed`, wb_ptr addresses the [L, h_out, r] stacks of the decode path (weights_b_t) - same result,
-    faster kernel."""
-    _native_module().sgmv_expand(y, v, wb_ptr, s_start, s_end, tmp, layer_idx, y_offset, y_slice_size, transposed)
+    faster kernel; `tiles` is then an optional row-tile plan of the segment tables (same result again)."""
+    _native_module().sgmv_expand(y, v, wb_ptr, s_start, s_end, tmp, layer_idx, y_offset, y_slice_size, transposed,
+                                 True, tiles)
 
 
 def segmented_matmul(

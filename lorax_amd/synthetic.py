@@ -112,6 +112,11 @@ def _splice_rank_group(rs, layer, rank: int, extra) -> None:
     rs.num_long_segments = n_long + len(extra)
     if rs.segments_key is not None:
         rs.segments_key = (rs.segments_key, tuple(extra))
+    # the row-tile plans name segments by their position in the tables: cut them again for the new tables
+    from lorax_amd.adapters import _tile_plans
+
+    rs.shrink_tiles, rs.expand_tiles = _tile_plans(rs.segment_starts.tolist(), rs.segment_ends.tolist(),
+                                                   rs.num_long_segments, rs.segment_starts.device)
 
 
 def _inject_segments(w: "Workload", batch: AdapterBatchData) -> None:

@@ -79,20 +79,27 @@ def test_sgmv_shrink_multi_validation():
     big = 8 * 1024 * 1024
     one = (_native.SgmvShrinkProblem * 1)(_native.SgmvShrinkProblem(P, P))
     two = (_native.SgmvShrinkProblem * 2)(_native.SgmvShrinkProblem(P, P), _native.SgmvShrinkProblem(P, P))
-    assert f(two, 0, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, 1, None) == EINVAL and "num_problems" in _err()
-    assert f(two, 5, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, 1, None) == EINVAL
-    assert f(None, 2, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, 1, None) == EINVAL
+    assert f(two, 0, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, None, 1, None) == EINVAL and "num_problems" in _err()
+    assert f(two, 5, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, None, 1, None) == EINVAL
+    assert f(None, 2, P, P, P, 2, 1000, 4096, 16, 0, 1.0, 1, P, big, None, 1, None) == EINVAL
     # stacked launch (2 x 64 <= 128, h_in a multiple of 128, more than 512 rows): its own checks
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 1, P, big - 1, 1, None) == ETMPSIZE
-    assert f(two, 2, P, P, P, 0, 1000, 4096, 64, 0, 1.0, 1, P, big, 1, None) == OK  # no segments
-    assert f(two, 2, P, P, None, 2, 1000, 4096, 64, 0, 1.0, 1, P, big, 1, None) == EINVAL and "null" in _err()
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, -1, 1.0, 1, P, big, 1, None) == EINVAL
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 1, P, big - 1, None, 1, None) == ETMPSIZE
+    assert f(two, 2, P, P, P, 0, 1000, 4096, 64, 0, 1.0, 1, P, big, None, 1, None) == OK  # no segments
+    assert f(two, 2, P, P, None, 2, 1000, 4096, 64, 0, 1.0, 1, P, big, None, 1, None) == EINVAL and "null" in _err()
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, -1, 1.0, 1, P, big, None, 1, None) == EINVAL
     # one launch per projection (summed rank 192; or a single projection): lorax_sgmv_shrink's checks
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 96, 0, 1.0, 1, P, big - 1, 1, None) == ETMPSIZE
-    assert f(one, 1, P, P, P, 2, 1000, 4100, 16, 0, 1.0, 1, P, big, 1, None) == ENOKERNEL
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 12, 0, 1.0, 1, P, big, 1, None) == ENOKERNEL
-    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 2, P, big, 1, None) == EINVAL and "accumulate" in _err()
-    assert f(two, 2, P, P, P, 0, 1000, 4096, 64, 0, 1.0, 0, P, 4 * big, 1, None) == OK  # a larger scratch is accepted
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 96, 0, 1.0, 1, P, big - 1, None, 1, None) == ETMPSIZE
+    assert f(one, 1, P, P, P, 2, 1000, 4100, 16, 0, 1.0, 1, P, big, None, 1, None) == ENOKERNEL
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 12, 0, 1.0, 1, P, big, None, 1, None) == ENOKERNEL
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 2, P, big, None, 1, None) == EINVAL and "accumulate" in _err()
+    assert f(two, 2, P, P, P, 0, 1000, 4096, 64, 0, 1.0, 0, P, 4 * big, None, 1, None) == OK  # a larger scratch is accepted
+    # a row-tile plan: records must be aligned, the height bound at least 1
+    bad = _native.SgmvTiles(P + 4, 3, 48)
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 1, P, big, ctypes.byref(bad), 1, None) == EINVAL and "tile plan" in _err()
+    bad = _native.SgmvTiles(P, 3, 0)
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 1, P, big, ctypes.byref(bad), 1, None) == EINVAL
+    empty = _native.SgmvTiles(P, 0, 16)  # a plan without tiles: nothing to do
+    assert f(two, 2, P, P, P, 2, 1000, 4096, 64, 0, 1.0, 1, P, big, ctypes.byref(empty), 1, None) == OK
 
 
 def test_sgmv_lora_multi_validation():
@@ -122,6 +129,49 @@ def test_sgmv_expand_validation():
         assert f(P, P, P, P, P, 2, 16, 16, 4096, layout, 0, 1 << 24, 0, 1, P, 120, 1, None) == EINVAL  # row pitch
         assert "2^24" in _err()
     assert f(P, P, P, P, P, 2, 16, 16, 4096, 2, 0, 4096, 0, 1, P, 120, 1, None) == EINVAL  # unknown layout
+
+
+def test_sgmv_expand_planned_validation():
+    f = _native.lib().lorax_sgmv_expand_planned
+    assert f(P, P, P, P, P, 0, 16, 16, 4096, 0, 4096, 0, 1, None, 1, None) == OK  # no segments
+    assert f(P, P, P, P, P, 2, 16, 12, 4096, 0, 4096, 0, 1, None, 1, None) == ENOKERNEL
+    assert f(P, P, P, P, None, 2, 16, 16, 4096, 0, 4096, 0, 1, None, 1, None) == EINVAL
+    bad = _native.SgmvTiles(P, -1, 256)
+    assert f(P, P, P, P, P, 2, 16, 16, 4096, 0, 4096, 0, 1, ctypes.byref(bad), 1, None) == EINVAL and "tile plan" in _err()
+    empty = _native.SgmvTiles(P, 0, 256)
+    assert f(P, P, P, P, P, 2, 16, 16, 4096, 0, 4096, 0, 1, ctypes.byref(empty), 1, None) == OK
+
+
+def test_plan_tiles_cuts_every_row_once():
+    """lorax_sgmv_plan_tiles (host only): every row of every non-empty segment in exactly one tile, tiles inside
+    their segment and no higher than the bound, numbered inside the segment; empty and negative segments get none."""
+    starts = [5, 100, 100, -1, 400, 2000]
+    ends = [47, 100, 90, -1, 1500, 2003]
+    T = 2500
+    for kind, limit in ((_native.TILES_SHRINK, 64), (_native.TILES_EXPAND, 256 + 32 + 16)):
+        records, tile_rows = _native.plan_tiles(starts, ends, T, kind)
+        assert tile_rows <= limit
+        covered = {}
+        last_index = {}
+        for seg, row0, row_end, index in records.tolist():
+            assert starts[seg] <= row0 < row_end <= ends[seg] and row_end - row0 <= tile_rows
+            assert index == last_index.get(seg, -1) + 1
+            last_index[seg] = index
+            for row in range(row0, row_end):
+                assert row not in covered
+                covered[row] = seg
+        want = {row: seg for seg, (s, e) in enumerate(zip(starts, ends)) for row in range(max(s, 0), min(e, T))}
+        assert covered == want
+    # bounds beyond the batch are clamped; a table without rows gives an empty plan
+    records, _ = _native.plan_tiles([10], [100], 50, _native.TILES_SHRINK)
+    assert records[:, 2].max() == 50
+    records, _ = _native.plan_tiles([3, -1], [3, -1], 50, _native.TILES_EXPAND)
+    assert records.shape == (0, 4)
+    # a thousand rows in ten segments: low tiles (the launch also cuts the hidden dimension); a long batch: 64 rows
+    records, tile_rows = _native.plan_tiles(list(range(0, 1000, 100)), list(range(100, 1100, 100)), 1000, _native.TILES_SHRINK)
+    assert tile_rows == 16 and len(records) == 70
+    records, tile_rows = _native.plan_tiles([0], [40000], 40000, _native.TILES_SHRINK)
+    assert tile_rows == 64 and len(records) == 625
 
 
 def test_python_binding_rejects_cpu_tensors():

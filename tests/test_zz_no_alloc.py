@@ -63,3 +63,27 @@ def test_static_shrink_matches_the_tmp_entry_point(r, h_in, first, second):
         assert_close(v, want, f"v lens={lens}")
 
 
+
+
+def test_static_shrink_refuses_a_split_that_does_not_fit_its_scratch():
+    """12 000 rows at rank 64 over h_in = 4160 are 189 row tiles of the register-operand kernel, which would split
+    the hidden dimension three ways: three fp32 copies of v (9.2 MB) exceed the 8 MiB array, so the call is refused
+    and nothing is launched; the entry point with a caller's tmp runs it with two."""
+    r, h_in, T = 64, 4160, 12000
+    x = torch.zeros((T, h_in), dtype=torch.bfloat16, device=DEV)
+    v = torch.full((T, r), 3.0, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros((1, r, h_in), dtype=torch.bfloat16, device=DEV)
+    s_start = torch.tensor([0], dtype=torch.int32, device=DEV)
+    s_end = torch.tensor([T], dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="static scratch"):
+        _native.sgmv_shrink_static(v, x, ptr_table([w], DEV), s_start, s_end, 0)
+    torch.cuda.synchronize()
+    assert torch.all(v == 3.0)
+    # a batch that does not split (more row tiles) has no limit: 20 000 rows use no scratch at all
+    T2 = 20000
+    x2 = torch.ones((T2, 1056), dtype=torch.bfloat16, device=DEV)
+    w2 = torch.ones((1, 128, 1056), dtype=torch.bfloat16, device=DEV)
+    v2 = torch.zeros((T2, 128), dtype=torch.bfloat16, device=DEV)
+    _native.sgmv_shrink_static(v2, x2, ptr_table([w2], DEV), s_start, torch.tensor([T2], dtype=torch.int32, device=DEV), 0)
+    torch.cuda.synchronize()
+    assert torch.all(v2 == 1056)
