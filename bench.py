@@ -48,7 +48,7 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
-    p.add_argument("--config", default="all", choices=["all", "1", "2", "3", "4", "5", "mid", "5dec"])
+    p.add_argument("--config", default="all", choices=["all", "1", "2", "3", "4", "5", "mid", "5dec", "2stk"])
     p.add_argument("--windows", type=int, default=5, help="timing windows of --steps steps per configuration")
     p.add_argument("--cpu-budget", type=float, default=0.0,
                    help="seconds of host time for the CPU baseline of one configuration (0 = the default share)")
@@ -69,9 +69,9 @@ def parse_args():
     return p.parse_args()
 
 
-DEFAULT_LAYERS = {"1": 32, "2": 32, "3": 8, "4": 2, "5": 1, "mid": 16, "5dec": 1}
+DEFAULT_LAYERS = {"1": 32, "2": 32, "3": 8, "4": 2, "5": 1, "mid": 16, "5dec": 1, "2stk": 32}
 # seconds of host time the CPU baseline of each configuration may take in the default run
-CPU_BUDGET_S = {"1": 2.0, "2": 5.0, "3": 5.0, "4": 6.0, "5": 6.0, "mid": 2.0, "5dec": 4.0}
+CPU_BUDGET_S = {"1": 2.0, "2": 5.0, "3": 5.0, "4": 6.0, "5": 6.0, "mid": 2.0, "5dec": 4.0, "2stk": 2.0}
 GATED = ("1", "2", "3", "4")  # configurations whose roofline fractions feed roofline_min
 
 
@@ -83,6 +83,13 @@ def build_workload(cfg: str, layers: int, device):
         return synthetic.mid_prefill(device, num_layers=L, weights_on_device=True)
     if cfg == "5dec":
         return synthetic.config5_decode(device, num_layers=L, weights_on_device=True)
+    if cfg == "2stk":
+        # configuration 2 served from stacked weights ([num_adapters, r, h] tensors per layer and projection,
+        # one entry number per token): the reference's path for preloaded adapters (utils/layers.py:79-105)
+        w = synthetic.config2(device, num_layers=L, weights_on_device=True)
+        w.name = "cfg2_bgmv_decode_qkvo_stacked_weights"
+        w.stacked = True
+        return w
     return synthetic.CONFIGS[int(cfg)](device, num_layers=L, weights_on_device=True)
 
 
@@ -111,6 +118,9 @@ class Plan:
         self.batch = w.batch_data()
         self.calls = []  # (kind, fn(layer), algorithmic bytes, flops, gather bytes: weights once per routed row)
         T = w.num_tokens
+        if getattr(w, "stacked", False):
+            self._add_stacked(w)
+            return
         for group in w.groups:
             x = w.inputs[group.name]
             y = torch.zeros((T, group.h_out), dtype=w.dtype, device=w.device)
@@ -296,6 +306,55 @@ class Plan:
             flops += 2 * rows * r * (h_in + size)
         self.calls.append(("sgmv_lora", lambda layer: _native.sgmv_lora_multi(problems, x, starts, ends, r, layer),
                            nbytes, flops, gather))
+
+    def _add_stacked(self, w):
+        """The decode step over stacked weights: per projection group one PunicaWrapper.add_lora_slices call, which
+        runs shrink and expand of the group's slices in one launch from the step's routing plan over stack entries.
+        Same algorithmic bytes as the pointer-table launches of the same batch."""
+        import torch
+
+        from lorax_amd.adapters import LORA, stack_preloaded_adapters
+        from lorax_amd.punica_wrapper import PunicaWrapper
+        from lorax_amd.synthetic import make_meta
+
+        e = 2
+        adapters = sorted(w.rank_of_adapter)
+        entry_of = {a: i for i, a in enumerate(adapters)}
+        stacks = stack_preloaded_adapters(w.weights, adapters, w.device)
+        wrapper = PunicaWrapper(max(w.num_tokens, 1), max(w.num_tokens, 1), str(w.device), enabled=True)
+        # adapter 0 is the base model on this path: entry i belongs to adapter index i + 1
+        wrapper.update_metadata(make_meta([entry_of[a] + 1 if a in entry_of else 0 for a in w.adapter_indices],
+                                          w.device), prefill=False)
+        self.keep = (stacks, wrapper)
+        T = w.num_tokens
+        for group in w.groups:
+            x = w.inputs[group.name]
+            y = torch.zeros((T, group.h_out), dtype=w.dtype, device=w.device)
+            nbytes = gather = flops = 0
+            x_counted = False
+            off = 0
+            spans = []
+            for name, size in zip(group.layer_names, group.sizes):
+                data = self.batch.data.get(name, {}).get(LORA)
+                spans.append((name, off, size))
+                off += size
+                if data is None:
+                    continue
+                for r, rd in data.rank_data.items():
+                    n, u = self._bgmv_counts(rd)
+                    if not x_counted:
+                        routed = int(sum(1 for a in w.adapter_indices if a in entry_of))
+                        nbytes += routed * group.h_in * e
+                        gather += routed * group.h_in * e
+                        x_counted = True
+                    nbytes += u * r * (group.h_in + size) * e + 2 * n * size * e
+                    gather += n * r * (group.h_in + size) * e + 2 * n * size * e
+                    flops += 2 * n * r * (group.h_in + size)
+
+            def step(layer, x=x, y=y, spans=spans):
+                wrapper.add_lora_slices(y, x, [stacks[(name, layer)] + (first, size) for name, first, size in spans], 1.0)
+
+            self.calls.append(("bgmv_lora", step, nbytes, flops, gather))
 
     def _add_bgmv_reference(self, x, y, off, size, h_in, r, rd):
         import torch
@@ -692,7 +751,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    todo = ["2", "1", "3", "4", "5", "mid", "5dec"] if args.config == "all" else [args.config]
+    todo = ["2", "1", "3", "4", "5", "mid", "5dec", "2stk"] if args.config == "all" else [args.config]
     records = {}
     for cfg in todo:
         print(f"bench: configuration {cfg}", file=sys.stderr, flush=True)
@@ -728,8 +787,9 @@ def main():
         "ceiling": ceiling,
     }
     if args.config == "all":
-        out["configs"] = {f"cfg{k}": compact(records[k]) for k in todo if k not in ("mid", "5dec")}
-        out["extra"] = {"mid_prefill_1k": compact(records["mid"]), "cfg5_decode_tokens_bgmv": compact(records["5dec"])}
+        out["configs"] = {f"cfg{k}": compact(records[k]) for k in todo if k not in ("mid", "5dec", "2stk")}
+        out["extra"] = {"mid_prefill_1k": compact(records["mid"]), "cfg5_decode_tokens_bgmv": compact(records["5dec"]),
+                        "cfg2_stacked_weights": compact(records["2stk"])}
         fracs = [(f"cfg{k}", kind, rec["frac"], records[k]["roofline"]["bound"])
                  for k in GATED for kind, rec in records[k]["kernels"].items()]
         lowest = min(fracs, key=lambda t: t[2])

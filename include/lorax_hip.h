@@ -110,6 +110,13 @@ int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* ind
  * A record whose word [0] is 0 is padding and is skipped, so a plan can be kept at a fixed number of
  * records for graph replay (the reference pads its tables the same way, utils/graph.py:71-73,421-425).
  * With a plan, w_ptrs and indices are not read and may be NULL.
+ *
+ * Stacked weights.  The reference's newer path keeps preloaded adapters in ONE tensor per layer and projection,
+ * lora_a [num_adapters, r, h_in] and lora_b [num_adapters, h_out, r] (lorax_server/models/model.py:289-334,
+ * utils/punica.py:689-748), and routes with an entry number per token.  A planned problem serves it directly:
+ * with a_stack (shrink launches) / b_stack (expand launches) set to the tensor's base address, plan words [5] and
+ * [6] hold the adapter's ENTRY NUMBER instead of an address, layer_idx must be 0, and one plan - built once per
+ * batch from the per-token entry numbers - serves every layer and projection.
  */
 typedef struct lorax_bgmv_problem {
   void* y;                /* [num_tokens, y_stride] output                         */
@@ -122,6 +129,8 @@ typedef struct lorax_bgmv_problem {
   const int64_t* plan;    /* optional routing plan (see above), else NULL          */
   int32_t num_groups;     /* records in plan                                       */
   int32_t h_in;           /* this problem's input width; 0 = the call's h_in       */
+  const void* a_stack;    /* stacked weights (see above), else NULL                */
+  const void* b_stack;
 } lorax_bgmv_problem_t;
 
 int lorax_bgmv_multi(const lorax_bgmv_problem_t* problems, int32_t num_problems, int64_t num_tokens,
@@ -231,11 +240,12 @@ typedef struct lorax_sgmv_tiles {
  * Builds a tile plan on the HOST: s_start / s_end are host copies of the segment tables of the launch (empty and
  * negative segments get no tile, bounds are clamped to [0, num_tokens]).  Writes up to `capacity` records to
  * `tiles` (host memory; the caller uploads them), the number of records to *num_tiles and the bound of their
- * heights to *tile_rows.  Returns LORAX_ESPACE, with *num_tiles set, when capacity is too small (or tiles NULL).
+ * heights to *tile_rows.  `rank` is the LoRA rank of the launch (shrink tiles are not made lower than a quarter
+ * of it; 0 = unknown).  Returns LORAX_ESPACE, with *num_tiles set, when capacity is too small (or tiles NULL).
  */
 int lorax_sgmv_plan_tiles(const int32_t* s_start, const int32_t* s_end, int32_t num_segments, int64_t num_tokens,
-                          int32_t kind, lorax_sgmv_tile_t* tiles, int32_t capacity, int32_t* num_tiles,
-                          int32_t* tile_rows);
+                          int32_t kind, int32_t rank, lorax_sgmv_tile_t* tiles, int32_t capacity,
+                          int32_t* num_tiles, int32_t* tile_rows);
 
 /*
  * SGMV shrink of up to 4 projections that share x, the segments and the rank (q/k/v, gate/up), LORAX_A_RH

@@ -40,6 +40,8 @@ class BgmvProblem(ctypes.Structure):
         ("plan", _c.c_void_p),
         ("num_groups", _c.c_int32),
         ("h_in", _c.c_int32),
+        ("a_stack", _c.c_void_p),
+        ("b_stack", _c.c_void_p),
     ]
 
 
@@ -149,7 +151,7 @@ _SIGNATURES = {
     ),
     "lorax_sgmv_plan_tiles": (
         _c.c_int,
-        [_c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64, _c.c_int32, _c.c_void_p, _c.c_int32,
+        [_c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_int64, _c.c_int32, _c.c_int32, _c.c_void_p, _c.c_int32,
          _c.POINTER(_c.c_int32), _c.POINTER(_c.c_int32)],
     ),
     "lorax_set_fixed_order_shrink": (_c.c_int, [_c.c_int32]),
@@ -307,13 +309,15 @@ def bgmv(y, x, w_ptr, indicies, layer_idx, scale, y_offset=0, y_slice_size=None)
 PLAN_RECORD_WORDS = 8
 
 
-def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> None:
+def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None, stacks=None) -> None:
     """lorax_bgmv_multi: `problems` is a list of up to 16 tuples (y, x, w_ptr, indicies, y_offset, y_slice_size)
     that share the token count and the direction; shrink problems share x.shape and may differ in rank
     (y's width), expand problems may differ in rank (x's width) and output width.  y_slice_size None means
     the whole width of y.
     `plans`, if given, holds one routing plan per problem: an int64 device tensor [num_groups, 8]; w_ptr and
-    indicies of a planned problem may then be None (the kernels read the plan only)."""
+    indicies of a planned problem may then be None (the kernels read the plan only).
+    `stacks` (with plans): per problem the stacked weight tensor [num_adapters, rows, cols] whose entry numbers the
+    plan's address words hold - lora_a stacks for a shrink launch, lora_b stacks for an expand launch."""
     if not 1 <= len(problems) <= MAX_BGMV_PROBLEMS:
         raise RuntimeError(f"between 1 and {MAX_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
     arr = (BgmvProblem * len(problems))()
@@ -347,9 +351,13 @@ def bgmv_multi(problems, layer_idx, scale=1.0, accumulate=True, plans=None) -> N
             plan_ptr, num_groups = plan.data_ptr(), plan.size(0)
             if num_groups == 0:
                 plan_ptr = x.data_ptr()  # an empty plan has no storage; any non-null address will do
+        stack = None
+        if stacks is not None and plans is not None:
+            _check_stack(stacks[i], x)
+            stack = stacks[i].data_ptr()
         arr[i] = BgmvProblem(y.data_ptr(), x.data_ptr(), None if planned_only else w_ptr.data_ptr(),
                              None if planned_only else indicies.data_ptr(), int(y_offset),
-                             y.size(1), h_out, plan_ptr, num_groups, x.size(1))
+                             y.size(1), h_out, plan_ptr, num_groups, x.size(1), stack, stack)
     with torch.cuda.device(x0.device):
         rc = lib().lorax_bgmv_multi(arr, len(problems), x0.size(0), x0.size(1), int(layer_idx), float(scale),
                                     1 if accumulate else 0, _dtype_code(x0), _stream(x0))
@@ -370,9 +378,18 @@ def bgmv_lora_fits(rank: int, h_in: int, h_out: int) -> bool:
     return rank * h_in * 2 <= 128 * 1024 and h_out <= (256 // (rank // 8)) * 16
 
 
-def bgmv_lora_multi(problems, rank, layer_idx, scale=1.0) -> None:
+def _check_stack(stack, x) -> None:
+    if not isinstance(stack, torch.Tensor) or stack.dim() != 3 or not stack.is_contiguous() or stack.dtype != x.dtype \
+            or stack.device != x.device:
+        raise RuntimeError("stacked weights must be a contiguous [num_adapters, rows, cols] tensor of the input's "
+                           "dtype on its device")
+
+
+def bgmv_lora_multi(problems, rank, layer_idx, scale=1.0, stacks=None) -> None:
     """lorax_bgmv_lora_multi: `problems` is a list of up to 4 tuples (y, x, plan, y_offset, y_slice_size) that
-    share x.shape; y[:, window] += (x @ A^T) @ B^T per planned token chunk, rank 8 or 16."""
+    share x.shape; y[:, window] += (x @ A^T) @ B^T per planned token chunk, rank 8 or 16.
+    `stacks`: per problem a pair (lora_a [num_adapters, r, h_in], lora_b [num_adapters, h_out, r]) of stacked weight
+    tensors; the plan's address words then hold entry numbers and layer_idx must be 0."""
     if not 1 <= len(problems) <= MAX_FUSED_BGMV_PROBLEMS:
         raise RuntimeError(f"between 1 and {MAX_FUSED_BGMV_PROBLEMS} problems per launch, got {len(problems)}")
     arr = (BgmvProblem * len(problems))()
@@ -390,8 +407,18 @@ def bgmv_lora_multi(problems, rank, layer_idx, scale=1.0) -> None:
             raise RuntimeError(f"plan must be an int64 [num_groups, {PLAN_RECORD_WORDS}] tensor on the device of x")
         h_out = y.size(1) if y_slice_size is None else int(y_slice_size)
         plan_ptr = plan.data_ptr() if plan.size(0) > 0 else x.data_ptr()
+        a_stack = b_stack = None
+        if stacks is not None:
+            if int(layer_idx) != 0:
+                raise RuntimeError("stacked weights hold one layer: layer_idx must be 0")
+            _check_stack(stacks[i][0], x)
+            _check_stack(stacks[i][1], x)
+            if stacks[i][0].shape[1:] != (rank, x.size(1)) or stacks[i][1].shape[1:] != (h_out, rank):
+                raise RuntimeError(f"stacked weights of problem {i} do not have the shapes [n, {rank}, {x.size(1)}] "
+                                   f"and [n, {h_out}, {rank}]")
+            a_stack, b_stack = stacks[i][0].data_ptr(), stacks[i][1].data_ptr()
         arr[i] = BgmvProblem(y.data_ptr(), x.data_ptr(), None, None, int(y_offset), y.size(1), h_out, plan_ptr,
-                             plan.size(0))
+                             plan.size(0), 0, a_stack, b_stack)
     with torch.cuda.device(x0.device):
         rc = lib().lorax_bgmv_lora_multi(arr, len(problems), x0.size(0), x0.size(1), int(rank), int(layer_idx),
                                          float(scale), _dtype_code(x0), _stream(x0))
@@ -531,9 +558,9 @@ def sgmv_shrink_multi(ys, x, w_ptrs, s_start, s_end, tmp, layer_idx, scale: floa
         _raise_last(rc)
 
 
-def plan_tiles(s_start, s_end, num_tokens: int, kind: int):
+def plan_tiles(s_start, s_end, num_tokens: int, kind: int, rank: int = 0):
     """lorax_sgmv_plan_tiles on host copies of the segment tables (sequences of int): returns (records as a numpy
-    int32 [num_tiles, 4] array, tile_rows)."""
+    int32 [num_tiles, 4] array, tile_rows).  `rank`: the LoRA rank of the launch, 0 = unknown."""
     import numpy as np
 
     starts = np.ascontiguousarray(s_start, dtype=np.int32)
@@ -545,7 +572,8 @@ def plan_tiles(s_start, s_end, num_tokens: int, kind: int):
     while True:
         records = np.empty((capacity, 4), dtype=np.int32)
         rc = lib().lorax_sgmv_plan_tiles(starts.ctypes.data, ends.ctypes.data, starts.shape[0], int(num_tokens),
-                                         int(kind), records.ctypes.data, capacity, ctypes.byref(n), ctypes.byref(rows))
+                                         int(kind), int(rank), records.ctypes.data, capacity, ctypes.byref(n),
+                                         ctypes.byref(rows))
         if rc == ESPACE:
             capacity = int(n.value)
             continue

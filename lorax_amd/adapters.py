@@ -310,7 +310,7 @@ def _segment_order(segs: List[int], seg_adapters: List[int], bounds: List[int], 
                       seg_adapters[s])
 
 
-def _tile_plans(starts: List[int], ends: List[int], num_long: int, device):
+def _tile_plans(starts: List[int], ends: List[int], num_long: int, device, rank: int = 0):
     """Row-tile plans (shrink, expand) of the first num_long segments, cut by the library's host routine and
     uploaded; (None, None) where the library is not loaded or the tables live on the CPU."""
     from lorax_amd import _native
@@ -320,7 +320,7 @@ def _tile_plans(starts: List[int], ends: List[int], num_long: int, device):
     rows = max(ends[:num_long], default=0)
     plans = []
     for kind in (_native.TILES_SHRINK, _native.TILES_EXPAND):
-        records, tile_rows = _native.plan_tiles(starts[:num_long], ends[:num_long], rows, kind)
+        records, tile_rows = _native.plan_tiles(starts[:num_long], ends[:num_long], rows, kind, rank)
         plans.append(_native.TilePlan(torch.from_numpy(records.copy()).to(device), tile_rows))
     return plans[0], plans[1]
 
@@ -482,7 +482,7 @@ class BatchLoraWeights(BatchAdapterWeights):
                 shrink_tiles, expand_tiles = _tile_plans(
                     [head_starts[s] if head_starts is not None else seg_bounds[s] for s in segs],
                     [head_ends[s] if head_starts is not None else seg_bounds[s + 1] for s in segs],
-                    num_long if num_long is not None else len(segs), device)
+                    num_long if num_long is not None else len(segs), device, rank)
             else:
                 # slot of an adapter = position of its first segment inside this group's pointer slice
                 slot: Dict[int, int] = {}

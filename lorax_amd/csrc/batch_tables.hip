@@ -225,7 +225,7 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
           const std::vector<lorax::SegmentSpan> live =
               lorax::live_segments(tile_starts.data(), tile_ends.data(), desc.num_long_segments, num_tokens);
           tile_buf.clear();
-          desc.shrink_tile_rows = lorax::plan_shrink_tiles(live, tile_buf);
+          desc.shrink_tile_rows = lorax::plan_shrink_tiles(live, tile_buf, desc.rank, lorax::tuning().shrink_rows);
           desc.num_shrink_tiles = static_cast<int32_t>(tile_buf.size());
           desc.shrink_tiles_off = pack.reserve(static_cast<int64_t>(tile_buf.size()) * sizeof(lorax_sgmv_tile_t));
           if (lorax_sgmv_tile_t* out = pack.at<lorax_sgmv_tile_t>(desc.shrink_tiles_off))
@@ -300,15 +300,16 @@ extern "C" int lorax_build_batch_tables(const int64_t* adapter_indices, int64_t 
 }
 
 extern "C" int lorax_sgmv_plan_tiles(const int32_t* s_start, const int32_t* s_end, int32_t num_segments,
-                                     int64_t num_tokens, int32_t kind, lorax_sgmv_tile_t* tiles, int32_t capacity,
-                                     int32_t* num_tiles, int32_t* tile_rows) {
+                                     int64_t num_tokens, int32_t kind, int32_t rank, lorax_sgmv_tile_t* tiles,
+                                     int32_t capacity, int32_t* num_tiles, int32_t* tile_rows) {
   if (num_segments < 0 || num_tokens < 0 || num_tiles == nullptr || tile_rows == nullptr ||
       (num_segments > 0 && (s_start == nullptr || s_end == nullptr)) ||
       (kind != LORAX_TILES_SHRINK && kind != LORAX_TILES_EXPAND))
     return LORAX_EINVAL;
   const std::vector<lorax::SegmentSpan> live = lorax::live_segments(s_start, s_end, num_segments, num_tokens);
   std::vector<lorax_sgmv_tile_t> out;
-  *tile_rows = kind == LORAX_TILES_SHRINK ? lorax::plan_shrink_tiles(live, out) : lorax::plan_expand_tiles(live, out);
+  *tile_rows = kind == LORAX_TILES_SHRINK ? lorax::plan_shrink_tiles(live, out, rank, lorax::tuning().shrink_rows)
+                                          : lorax::plan_expand_tiles(live, out);
   *num_tiles = static_cast<int32_t>(out.size());
   if (tiles == nullptr || static_cast<size_t>(capacity < 0 ? 0 : capacity) < out.size()) return out.empty() ? LORAX_OK : LORAX_ESPACE;
   std::copy(out.begin(), out.end(), tiles);

@@ -206,6 +206,11 @@ __device__ __forceinline__ int resolve_chunk(const BgmvProblem& P, const int64_t
 #pragma unroll
     for (int g = 0; g < kGroup; ++g) toks[g] = static_cast<int>(rec[1 + g]);
     stack_addr = rec[expand ? 6 : 5];
+    // Stacked weights ([num_adapters, r, h_in] / [num_adapters, h_out, r] tensors, one entry per adapter): the
+    // record names the entry, not its address; a planned problem carries the tensors' bases in the table fields
+    // it has no other use for.
+    const int64_t base = expand ? reinterpret_cast<int64_t>(P.indices) : reinterpret_cast<int64_t>(P.w_ptrs);
+    if (base != 0) stack_addr = base + stack_addr * P.narrow * static_cast<int64_t>(P.width) * 2;
     return n;
   }
   int64_t idx;
@@ -861,8 +866,13 @@ __global__ __launch_bounds__(kBgmvThreads) void bgmv_lora_kernel(const BgmvBatch
   int toks[kGroup];
 #pragma unroll
   for (int g = 0; g < kGroup; ++g) toks[g] = static_cast<int>(rec[1 + g]);
-  const E* A = reinterpret_cast<const E*>(rec[5]) + layer_idx * R * static_cast<int64_t>(h_in);
-  const E* B = reinterpret_cast<const E*>(rec[6]) + layer_idx * h_out * static_cast<int64_t>(R);
+  // (stacked weights: the record names the adapter's entry of the [num_adapters, R, h_in] / [num_adapters, h_out, R]
+  // tensors whose bases the problem carries, see resolve_chunk)
+  const int64_t a_base = reinterpret_cast<int64_t>(P.w_ptrs), b_base = reinterpret_cast<int64_t>(P.indices);
+  const int64_t a_addr = a_base != 0 ? a_base + rec[5] * R * static_cast<int64_t>(h_in) * 2 : rec[5];
+  const int64_t b_addr = b_base != 0 ? b_base + rec[6] * R * static_cast<int64_t>(h_out) * 2 : rec[6];
+  const E* A = reinterpret_cast<const E*>(a_addr) + layer_idx * R * static_cast<int64_t>(h_in);
+  const E* B = reinterpret_cast<const E*>(b_addr) + layer_idx * h_out * static_cast<int64_t>(R);
   E* Y = static_cast<E*>(P.y);
   const E* X = static_cast<const E*>(P.x);
   // A narrow projection batched with wide ones (k and v next to q) fills one expand block only: it runs the

@@ -156,8 +156,13 @@ int bgmv_batch(const lorax_bgmv_problem_t* problems, int32_t count, int64_t num_
     if (a.expand && h_out > a.wide_max) a.wide_max = h_out;
     if (narrow > a.narrow) a.narrow = narrow;
     a.narrow_sum += narrow;
-    a.batch.p[i] =
-        BgmvProblem{q.y, q.x, q.w_ptrs, q.indices, q.y_offset, q.y_stride, wide, narrow, q.plan, q.num_groups};
+    // a planned problem reads neither table; its stacked-weight base (if any) travels in the field of the
+    // direction's table instead (bgmv.hip: resolve_chunk)
+    const int64_t* tab_a = planned ? static_cast<const int64_t*>(expand ? nullptr : q.a_stack) : q.w_ptrs;
+    const int64_t* tab_b = planned ? static_cast<const int64_t*>(expand ? q.b_stack : nullptr) : q.indices;
+    if (planned && ((expand ? q.b_stack : q.a_stack) != nullptr) && !aligned16(expand ? q.b_stack : q.a_stack))
+      return fail(LORAX_EINVAL, "stacked weights must be 16-byte aligned (problem %d)", i);
+    a.batch.p[i] = BgmvProblem{q.y, q.x, tab_a, tab_b, q.y_offset, q.y_stride, wide, narrow, q.plan, q.num_groups};
   }
   if (!planned) a.grid_rows = num_tokens;
   a.work_rows = planned ? a.grid_rows : (num_tokens + 1) / 2;
@@ -299,7 +304,7 @@ int lorax_bgmv(void* y, const void* x, const int64_t* w_ptrs, const int64_t* ind
                int64_t num_tokens, int32_t h_in, int32_t h_out, int64_t y_offset,
                int64_t y_stride, int64_t layer_idx, float scale, int32_t dtype, void* stream) {
   if (num_tokens == 0) return LORAX_OK;
-  const lorax_bgmv_problem_t one{y, x, w_ptrs, indices, y_offset, y_stride, h_out, nullptr, 0, 0};
+  const lorax_bgmv_problem_t one{y, x, w_ptrs, indices, y_offset, y_stride, h_out, nullptr, 0, 0, nullptr, nullptr};
   return bgmv_batch(&one, 1, num_tokens, h_in, layer_idx, scale, 1, dtype, stream);
 }
 
@@ -487,7 +492,10 @@ int lorax_bgmv_lora_multi(const lorax_bgmv_problem_t* problems, int32_t num_prob
                   (long long)q.y_stride, q.h_out);
     if (q.num_groups > a.grid_rows) a.grid_rows = q.num_groups;
     if (q.h_out > a.wide_max) a.wide_max = q.h_out;
-    a.batch.p[i] = BgmvProblem{q.y, q.x, nullptr, nullptr, q.y_offset, q.y_stride, q.h_out, r, q.plan, q.num_groups};
+    if ((q.a_stack == nullptr) != (q.b_stack == nullptr) || !aligned16(q.a_stack) || !aligned16(q.b_stack))
+      return fail(LORAX_EINVAL, "a_stack and b_stack go together and must be 16-byte aligned (problem %d)", i);
+    a.batch.p[i] = BgmvProblem{q.y,        q.x,        static_cast<const int64_t*>(q.a_stack), static_cast<const int64_t*>(q.b_stack),
+                               q.y_offset, q.y_stride, q.h_out, r, q.plan, q.num_groups};
   }
   if (a.grid_rows == 0) return LORAX_OK;
   const hipError_t e = launch_bgmv_lora(a, static_cast<hipStream_t>(stream));

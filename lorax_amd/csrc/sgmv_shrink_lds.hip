@@ -327,8 +327,7 @@ static LdsLaunch lds_launch_shape(const SgmvArgs& a, size_t room) {
   const int NB = (a.d_out + 15) / 16;
   LdsLaunch l{};
   const bool kslices_pref = tuning().shrink_lds != 2;
-  l.planned = a.tiles != nullptr && a.num_tiles > 0 && a.tile_rows >= 1 && a.tile_rows <= 64 && tuning().shrink_mb == 0 &&
-              tuning().shrink_rows == 0;
+  l.planned = a.tiles != nullptr && a.num_tiles > 0 && a.tile_rows >= 1 && a.tile_rows <= 64 && tuning().shrink_mb == 0;
   if (l.planned) {
     // the plan's tiles in buffers just high enough; the waves take k slices wherever that variant exists
     l.mblk = (a.tile_rows + 15) / 16;
@@ -372,7 +371,7 @@ static LdsLaunch lds_launch_shape(const SgmvArgs& a, size_t room) {
   }
   // K parts: a workgroup streams its tile's x and A at about 50 GB/s whatever the launch, so a launch of a
   // hundred tiles (a prefill batch of one or two thousand rows) leaves most of the chip idle.  Its hidden
-  // dimension is cut into parts of at least 8 stages and a second small launch adds the parts.  Up to 120 tiles:
+  // dimension is cut into parts of at least 8 stages and a second small launch adds the parts.  Up to 128 tiles:
   // about one workgroup per CU (two measured no faster).  Up to 192 tiles (a single long run of a few thousand
   // rows cut into 32-row tiles): two or three parts, about two workgroups per CU - measured on a 4096-row run at
   // rank 128, 140 tiles: 51 -> 40 us over h_in = 8192 and 145 -> 86 us over h_in = 28672 with three parts (two: 45
@@ -383,9 +382,10 @@ static LdsLaunch lds_launch_shape(const SgmvArgs& a, size_t room) {
   const int nst_all = a.d_in / kLdsKc;
   l.kparts = 1;
   if (a.partials != nullptr && !fixed_order_shrink() && (l.tiles < 192 || tuning().shrink_ksplit > 0)) {
-    // (121 to 170 tiles: three parts - a 4096-row run in exactly 128 tiles measured 45 us in two parts, 40 us in three)
+    // (a 4096-row run at rank 128 planned as exactly 128 tiles: 41 us in two parts, one workgroup per CU, against
+    // 48 us in three)
     const int64_t nt = l.tiles > 0 ? l.tiles : 1;
-    int kparts = static_cast<int>(nt <= 120 ? 256 / nt : (512 / nt < 3 ? 512 / nt : 3));
+    int kparts = static_cast<int>(nt <= 128 ? 256 / nt : 512 / nt);
     if (kparts > 8) kparts = 8;
     if (kparts > nst_all / 8) kparts = nst_all / 8;
     if (tuning().shrink_ksplit > 0) kparts = tuning().shrink_ksplit < nst_all ? tuning().shrink_ksplit : nst_all;

@@ -155,6 +155,34 @@ def bgmv_expand(
     bgmv_expand_slice(inputs, lora_b_weights, output_tensor, lora_indices_tensor, 0, width, add_inputs)
 
 
+def build_slot_plan(slots) -> "torch.Tensor":
+    """Routing plan (host, int64 [chunks, 8]) of a decode batch over STACKED weights: `slots` holds every token's
+    entry number in the stacked tensors, negative = no adapter.  One record per chunk of up to four tokens of one
+    entry: [count, four token rows (unused ones repeat the first), entry, entry, 0] - the records of
+    lorax_bgmv_multi with entry numbers where a pointer-table plan holds addresses, so ONE plan serves every layer
+    and projection of the step."""
+    import numpy as np
+
+    slots = np.asarray(slots, dtype=np.int64).reshape(-1)
+    routed = np.nonzero(slots >= 0)[0]
+    n = routed.shape[0]
+    if n == 0:
+        return torch.zeros((0, _native.PLAN_RECORD_WORDS), dtype=torch.int64)
+    order = routed[np.argsort(slots[routed], kind="stable")]  # grouped by entry, token order inside a group
+    entry = slots[order]
+    pos = np.arange(n)
+    starts = np.r_[True, entry[1:] != entry[:-1]]
+    rank = pos - np.maximum.accumulate(np.where(starts, pos, 0))  # position inside the entry's group
+    heads = rank % 4 == 0
+    chunk = np.cumsum(heads) - 1
+    records = np.zeros((int(chunk[-1]) + 1, _native.PLAN_RECORD_WORDS), dtype=np.int64)
+    records[:, 0] = np.bincount(chunk)
+    records[:, 1:5] = order[heads][:, None]
+    records[chunk, 1 + rank % 4] = order
+    records[:, 5] = records[:, 6] = entry[heads]
+    return torch.from_numpy(records)
+
+
 @torch.inference_mode()
 def bgmv_lora_slices(
     inputs: torch.Tensor,
@@ -162,13 +190,18 @@ def bgmv_lora_slices(
     output_tensor: torch.Tensor,
     lora_indices_tensor: torch.Tensor,
     scaling: float = 1.0,
+    plan: Optional[torch.Tensor] = None,
 ):
     """bgmv_shrink followed by bgmv_expand_slice(add_inputs=True) for several column slices of output_tensor that
     share `inputs` (q/k/v, gate/up): `slices` is a sequence of (lora_a_weights, lora_b_weights, slice_offset,
     slice_size), ranks may differ.  No counterpart among the reference's operators, which its wrapper calls once
     per slice (punica.py:750-773); here the shrinks of up to 16 slices are one launch and their expands another,
     and the intermediate is kept in the type of `inputs` and never zero-filled (the shrink overwrites the rows
-    of routed tokens and the expand reads no others)."""
+    of routed tokens and the expand reads no others).
+    `plan`: the batch's routing plan over stack entries (build_slot_plan of lora_indices_tensor, on the device).
+    With it no workgroup scans lora_indices_tensor, and slices of rank 8 or 16 with a small A slab run shrink and
+    expand in ONE launch per rank (scaling 1 only: that kernel scales the update, the two-launch path the
+    intermediate, and only at 1 do both round alike)."""
     assert inputs.dtype in (torch.float16, torch.bfloat16)
     assert inputs.is_contiguous() and output_tensor.is_contiguous()
     assert inputs.size(0) == output_tensor.size(0)
@@ -178,7 +211,17 @@ def bgmv_lora_slices(
         b = _stacked(lora_b_weights, "lora_b_weights")
         assert a.dtype == inputs.dtype and b.dtype == inputs.dtype
         assert inputs.size(1) == a.size(-1) and a.size(-2) == b.size(-1) and slice_size == b.size(-2)
-        jobs.append((stack_table(a), stack_table(b), a.size(-2), slice_offset, slice_size))
+        jobs.append((a, b, a.size(-2), slice_offset, slice_size))
+    if plan is not None and scaling == 1.0 and all(
+            _native.bgmv_lora_fits(r, inputs.size(1), size) for _, _, r, _, size in jobs):
+        step = _native.MAX_FUSED_BGMV_PROBLEMS
+        for rank in sorted({r for _, _, r, _, _ in jobs}):
+            same = [j for j in jobs if j[2] == rank]
+            for i in range(0, len(same), step):
+                chunk = same[i : i + step]
+                _native.bgmv_lora_multi([(output_tensor, inputs, plan, off, size) for _, _, _, off, size in chunk],
+                                        rank, 0, 1.0, stacks=[(a, b) for a, b, _, _, _ in chunk])
+        return
     step = _native.MAX_BGMV_PROBLEMS
     tokens = inputs.size(0)
     for i in range(0, len(jobs), step):
@@ -188,10 +231,17 @@ def bgmv_lora_slices(
         for _, _, r, _, _ in chunk:
             bufs.append(flat[pos : pos + tokens * r].view(tokens, r))
             pos += tokens * r
-        _native.bgmv_multi([(v, inputs, ta, lora_indices_tensor, 0, None) for v, (ta, _, _, _, _) in zip(bufs, chunk)],
-                           0, scaling, False)
-        _native.bgmv_multi([(output_tensor, v, tb, lora_indices_tensor, off, size)
-                            for v, (_, tb, _, off, size) in zip(bufs, chunk)], 0, 1.0, True)
+        if plan is not None:
+            plans = [plan] * len(chunk)
+            _native.bgmv_multi([(v, inputs, None, None, 0, None) for v in bufs], 0, scaling, False, plans,
+                               stacks=[a for a, _, _, _, _ in chunk])
+            _native.bgmv_multi([(output_tensor, v, None, None, off, size) for v, (_, _, _, off, size) in zip(bufs, chunk)],
+                               0, 1.0, True, plans, stacks=[b for _, b, _, _, _ in chunk])
+            continue
+        _native.bgmv_multi([(v, inputs, stack_table(a), lora_indices_tensor, 0, None)
+                            for v, (a, _, _, _, _) in zip(bufs, chunk)], 0, scaling, False)
+        _native.bgmv_multi([(output_tensor, v, stack_table(b), lora_indices_tensor, off, size)
+                            for v, (_, b, _, off, size) in zip(bufs, chunk)], 0, 1.0, True)
 
 
 @torch.inference_mode()

@@ -64,6 +64,10 @@ class PunicaWrapper:
         self._run_owners = torch.empty(max_batches, dtype=torch.int64, device=device)
         self._kernel_bounds: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
         self._max_length: Optional[int] = None
+        # decode: the batch's routing plan over stack entries (ops.build_slot_plan), one record per chunk of up
+        # to four tokens of one adapter, in a fixed buffer; _plan_records of them are in use
+        self._plan = torch.zeros((max_num_batched_tokens, 8), dtype=torch.int64, device=device)
+        self._plan_records: Optional[int] = None
 
     # ---- routing state ----------------------------------------------------------------------------
 
@@ -74,7 +78,16 @@ class PunicaWrapper:
         torch.sub(meta.adapter_indices, 1, out=self._token_lora_indices[:count])
         self.indices_len[0] = count
         self.is_prefill = bool(prefill)
+        self._plan_records = None
         if not prefill:
+            # Routing plan of the decode step: tokens grouped by adapter on the host (one copy of the indices
+            # down, as the table builder of the pointer-table path makes, and one copy of the records up), so
+            # that no workgroup of the step's launches scans the index tensor and the projections of rank 8 / 16
+            # run shrink and expand in one launch.
+            if self._token_lora_indices.is_cuda and count <= self._plan.size(0):
+                records = ops.build_slot_plan(meta.adapter_indices.detach().cpu().numpy() - 1)
+                self._plan[: records.size(0)].copy_(records, non_blocking=True)
+                self._plan_records = records.size(0)
             return
         bounds = getattr(meta, "adapter_segments", None)
         owners = getattr(meta, "segment_indices", None)
@@ -226,7 +239,8 @@ class PunicaWrapper:
                     and all(a.dtype == rows_x.dtype and b.dtype == rows_x.dtype for a, b, _, _ in slices))
         if together:
             if not self.is_prefill:
-                ops.bgmv_lora_slices(rows_x, slices, rows_y, self.token_lora_indices, scale)
+                plan = self._plan[: self._plan_records] if self._plan_records is not None else None
+                ops.bgmv_lora_slices(rows_x, slices, rows_y, self.token_lora_indices, scale, plan=plan)
             elif not self.no_lora:
                 starts, ends = self._kernel_bounds
                 ops.sgmv_lora_slices(rows_x, slices, rows_y, starts, ends - starts, self._run_owners[: self.batch_size],

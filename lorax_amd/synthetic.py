@@ -116,7 +116,7 @@ def _splice_rank_group(rs, layer, rank: int, extra) -> None:
     from lorax_amd.adapters import _tile_plans
 
     rs.shrink_tiles, rs.expand_tiles = _tile_plans(rs.segment_starts.tolist(), rs.segment_ends.tolist(),
-                                                   rs.num_long_segments, rs.segment_starts.device)
+                                                   rs.num_long_segments, rs.segment_starts.device, rank)
 
 
 def _inject_segments(w: "Workload", batch: AdapterBatchData) -> None:

@@ -172,6 +172,10 @@ def test_plan_tiles_cuts_every_row_once():
     assert tile_rows == 16 and len(records) == 70
     records, tile_rows = _native.plan_tiles([0], [40000], 40000, _native.TILES_SHRINK)
     assert tile_rows == 64 and len(records) == 625
+    # tiles are not lowered below a quarter of the rank: 4096 rows at rank 128 stay at 32 rows (128 tiles), at rank
+    # 64 they go down to 16 (256 tiles, one per CU)
+    assert _native.plan_tiles([0], [4096], 4096, _native.TILES_SHRINK, 128)[1] == 32
+    assert _native.plan_tiles([0], [4096], 4096, _native.TILES_SHRINK, 64)[1] == 16
 
 
 def test_python_binding_rejects_cpu_tensors():

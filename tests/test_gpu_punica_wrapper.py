@@ -194,3 +194,62 @@ def test_add_lora_packed_nslice(prefill, dtype, ranks, repeat):
         assert torch.equal(y.cpu(), y_each.cpu())  # same kernels, same arithmetic, one launch or three
     routed = torch.tensor(token_idx) >= 0
     assert torch.equal(y.cpu()[~routed], y0.cpu()[~routed])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("ranks,widths", [
+    ((8, 8, 8), (4096, 1024, 1024)),   # q/k/v at rank 8: shrink and expand in one launch
+    ((16, 16), (2048, 2048)),          # rank 16
+    ((8, 16, 8), (1024, 512, 512)),    # mixed 8 and 16: one launch per rank
+    ((32, 64, 8), (1024, 1024, 1024)),  # ranks beyond the single launch: two planned launches
+])
+def test_decode_with_a_slot_plan_equals_the_scanning_launches(dtype, ranks, widths):
+    """ops.bgmv_lora_slices with the batch's routing plan over stack entries (ops.build_slot_plan) against the same
+    call without it, bit for bit, and against the documented formula; PunicaWrapper.update_metadata builds the
+    plan and add_lora_slices uses it."""
+    print(f"case dtype={dtype} ranks={ranks} widths={widths}", flush=True)
+    gen = torch.Generator().manual_seed(sum(ranks))
+    T, h_in, n = 61, 4096, 7
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    total = sum(widths)
+    y0 = randn((T, total), 0.5, gen, dtype, DEV)
+    idx = torch.randint(-1, n, (T,), generator=gen)
+    idx[:9] = 3  # more than two chunks of one adapter
+    slices, off = [], 0
+    for r, w in zip(ranks, widths):
+        a, b = _stacks(n, r, h_in, w, gen, dtype)
+        slices.append((a, b, off, w))
+        off += w
+    plan_host = ops.build_slot_plan(idx.numpy())
+    # every routed token once, at most four per record, one entry per record
+    seen = []
+    for count, t0, t1, t2, t3, ea, eb, zero in plan_host.tolist():
+        rows = [t0, t1, t2, t3][:count]
+        assert 1 <= count <= 4 and ea == eb and zero == 0 and {int(idx[t]) for t in rows} == {ea}
+        seen += rows
+    assert sorted(seen) == [t for t in range(T) if idx[t] >= 0]
+    plan = plan_host.to(DEV)
+    y_scan, y_plan = y0.clone(), y0.clone()
+    ops.bgmv_lora_slices(x, slices, y_scan, idx.to(DEV), 1.0)
+    ops.bgmv_lora_slices(x, slices, y_plan, idx.to(DEV), 1.0, plan=plan)
+    torch.cuda.synchronize()
+    assert torch.equal(y_scan, y_plan)
+    y_ref = y0.cpu()
+    for a, b, first, w in slices:
+        y_ref = _ref_lora(y_ref, x.cpu(), a, b, idx.tolist(), 1.0, first, w, dtype)
+    assert_close(y_plan, y_ref, "planned decode", rounded=[(y_ref.float() - y0.cpu().float()).to(dtype)])
+    untouched = idx < 0
+    assert torch.equal(y_plan.cpu()[untouched], y0.cpu()[untouched])
+    # a scale other than 1 keeps the two-launch arithmetic (planned launches, same bits as the scanning ones)
+    y_a, y_b = y0.clone(), y0.clone()
+    ops.bgmv_lora_slices(x, slices, y_a, idx.to(DEV), 0.5)
+    ops.bgmv_lora_slices(x, slices, y_b, idx.to(DEV), 0.5, plan=plan)
+    assert torch.equal(y_a, y_b)
+    # through the wrapper: adapter 0 is the base model, entry i belongs to adapter i + 1
+    wrapper = PunicaWrapper(256, 64, DEV, enabled=True)
+    wrapper.update_metadata(make_meta((idx + 1).tolist(), torch.device(DEV)), prefill=False)
+    assert wrapper._plan_records == plan_host.size(0)
+    y_w = y0.clone()
+    wrapper.add_lora_slices(y_w, x, slices, 1.0)
+    torch.cuda.synchronize()
+    assert torch.equal(y_w, y_plan)
