@@ -268,8 +268,8 @@ int lorax_sgmv_plan_tiles(const int32_t* s_start, const int32_t* s_end, int32_t 
  * the hidden dimension into parts whose fp32 sums are added afterwards.  A call is deterministic, but the last
  * rounding of an element of v can differ between two batches that hold the same row (within the parity
  * tolerance by a wide margin: one spacing of dtype on a few percent of the elements).
- * lorax_set_fixed_order_shrink(1) gives that up for speed: every tile then walks from k = 0 and no launch cuts
- * the hidden dimension, so a row's result depends on nothing but the row and its adapter.
+ * lorax_set_fixed_order_shrink(1) trades speed for reproducibility: every tile then walks from k = 0 and no launch
+ * cuts the hidden dimension, so a row's result depends on nothing but the row and its adapter.
  */
 typedef struct {
   void* v;               /* [num_tokens, r] */

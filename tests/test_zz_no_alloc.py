@@ -87,3 +87,31 @@ def test_static_shrink_refuses_a_split_that_does_not_fit_its_scratch():
     _native.sgmv_shrink_static(v2, x2, ptr_table([w2], DEV), s_start, torch.tensor([T2], dtype=torch.int32, device=DEV), 0)
     torch.cuda.synchronize()
     assert torch.all(v2 == 1056)
+
+
+def test_static_shrink_inside_a_graph_capture():
+    """The entry point exists for callers under stream capture: after lorax_init a call is captured, the graph is
+    replayed three times with an eager call of lorax_sgmv_shrink in between, and every replay leaves the bits the
+    eager entry point computes (overwrite semantics are not offered here, so v is cleared inside the graph)."""
+    r, h_in, lens = 48, 2048, [700, 0, 41, 600]   # LDS-staged kernel, hidden dimension in parts: the scratch is used
+    x, stacks, table, s_start, s_end, starts, ends = _case(r, h_in, lens, 31)
+    _native.init(torch.device(DEV))
+    tmp = sgmv.get_tmp_tensor(torch.device(DEV))
+    v_ref = torch.zeros((x.size(0), r), dtype=x.dtype, device=DEV)
+    _native.sgmv_shrink(v_ref, x, table, s_start, s_end, tmp, 1)
+    v = torch.zeros_like(v_ref)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        v.zero_()  # a fill kernel, not a memset node
+        _native.sgmv_shrink_static(v, x, table, s_start, s_end, 1)
+    for replay in range(3):
+        v.fill_(5.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(v, v_ref), f"replay {replay}"
+        other = torch.zeros_like(v_ref)
+        _native.sgmv_shrink(other, x, table, s_start, s_end, tmp, 1)  # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(other, v_ref)
+    assert torch.count_nonzero(v) > 0
