@@ -38,6 +38,7 @@ def _plan(starts, ends, T, kind):
     (128, 1024, [1500]),                        # one long run
     (16, 4096, [5] * 40 + [300]),               # many short segments
     (24, 2752, [513, 17]),                      # a rank and a width that are not powers of two
+    (32, 512, [9, 300] * 50),                   # a hundred segments: table entries past the first 64
 ])
 def test_expand_with_a_plan_is_bit_identical(dtype, r, h_out, lens):
     print(f"case dtype={dtype} r={r} h_out={h_out} lens={lens}", flush=True)
@@ -74,6 +75,7 @@ def test_expand_with_a_plan_is_bit_identical(dtype, r, h_out, lens):
     (1, 128, 4096, [4096]),                        # one long run at rank 128
     (1, 40, 1536, [33] * 30),                      # a rank that is not a multiple of 16
     (3, 16, 512, [9000]),                          # many tiles: more than one round over the CUs
+    (2, 32, 1024, [70, 7] * 50),                   # a hundred segments: table entries past the first 64
 ])
 def test_shrink_with_a_plan(count, r, h_in, lens):
     print(f"case count={count} r={r} h_in={h_in} lens={lens}", flush=True)
