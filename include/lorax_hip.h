@@ -215,8 +215,9 @@ int lorax_sgmv_shrink_static(void* v, const void* x, const int64_t* w_ptrs, cons
  * number inside its segment.  Every row of every non-empty segment must be in exactly one tile, and no tile may
  * be higher than tile_rows.  lorax_sgmv_plan_tiles builds such a list from host copies of the tables (and
  * lorax_build_batch_tables emits one per rank group).  Records are clamped on the device to the call's
- * num_segments, num_tokens and tile_rows, so a wrong plan gives wrong results but touches no memory outside the
- * call's tensors.  The results do not depend on how a batch is cut into tiles, except that the shrink's last
+ * num_segments, num_tokens and tile_rows, and a tile whose segment has a null table entry is skipped, so a wrong
+ * plan gives wrong results but reads and writes x, v and y inside the call's bounds only (a tile may not name a
+ * segment whose table entry dangles: the entry is dereferenced, as it would be for a non-empty segment).  The results do not depend on how a batch is cut into tiles, except that the shrink's last
  * rounding can (its sums over the hidden dimension are added in an order that depends on the tile, see
  * lorax_sgmv_shrink_multi).
  */

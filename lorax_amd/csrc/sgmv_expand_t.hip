@@ -86,7 +86,9 @@ __global__ __launch_bounds__(kExpTThreads) void sgmv_expand_t_kernel(
     // small remainders are merged into the segment's other tiles: a tile's prologue (the search and the panel
     // operands) costs as much as a hundred rows
     if (!get_row_tile<true>(plan, s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
-    const E* BT = reinterpret_cast<const E*>(segment_entry(pre_w, W, rt.seg)) + layer_idx * h_out * static_cast<int64_t>(r);
+    const int64_t stack = segment_entry(pre_w, W, rt.seg);
+    if (plan.records != nullptr && stack == 0) break;  // a caller's plan that names a segment without a stack
+    const E* BT = reinterpret_cast<const E*>(stack) + layer_idx * h_out * static_cast<int64_t>(r);
     const int nmb = (rt.row_end - rt.row0 + 15) / 16;
 
     for (int pp = 0; pp < panels_per_wave; ++pp) {

@@ -120,12 +120,16 @@ __global__ __launch_bounds__(kLdsThreads) void sgmv_shrink_lds_kernel(
     if (!get_row_tile(plan, s_start, s_end, num_segments, num_tokens, rows_per_tile, tile, rt)) break;
     const E* A[kMaxShrinkGroup];
     int64_t stack0 = 0;
+    bool missing = false;
 #pragma unroll
     for (int p = 0; p < kMaxShrinkGroup; ++p) {
       const int64_t stack = segment_entry(pre_w[p], grp.w[p < grp.count ? p : 0], rt.seg);
       if (p == 0) stack0 = stack;
+      missing = missing || stack == 0;
       A[p] = reinterpret_cast<const E*>(stack) + layer_idx * r * static_cast<int64_t>(h_in);
     }
+    // (a caller's plan that names a segment without a stack: nothing to multiply; the search never yields one)
+    if (plan.records != nullptr && missing) break;
 
     // Source addresses of this thread's chunks.  Load j of a thread covers chunk id j * 256 + tid of
     // the tile: row = id / 16, position = id % 16, and it fetches the row's chunk position ^ (row & 15).

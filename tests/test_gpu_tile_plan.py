@@ -156,3 +156,45 @@ def test_batch_tables_carry_tile_plans_that_the_layer_uses():
     torch.cuda.synchronize()
     assert_close(with_plans, without.cpu(), "layer output with plans against without")
     assert torch.count_nonzero(with_plans) > 0
+
+
+def test_a_tile_that_names_a_segment_without_a_stack_is_skipped():
+    """A caller's plan may be wrong about a segment: a tile whose segment has a null table entry is dropped by both
+    kernels (and records are clamped to the call's sizes), the other tiles give the usual result."""
+    dtype, r, h_in, h_out, layer = torch.bfloat16, 32, 1024, 768, 0
+    gen = torch.Generator().manual_seed(9)
+    starts, ends, T = [0, 700, 700], [700, 700, 1300], 1300  # the middle segment is empty and has no stack
+    x = randn((T, h_in), 1.0, gen, dtype, DEV)
+    a = [randn((1, r, h_in), 0.05, gen, dtype, DEV), None, randn((1, r, h_in), 0.05, gen, dtype, DEV)]
+    bt = [randn((1, h_out, r), 0.05, gen, dtype, DEV), None, randn((1, h_out, r), 0.05, gen, dtype, DEV)]
+    s_start = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    s_end = torch.tensor(ends, dtype=torch.int32, device=DEV)
+    tmp = sgmv.get_tmp_tensor(torch.device(DEV))
+    tmp_e = sgmv.get_tmp_tensor_for_size(3, torch.device(DEV))
+    for kind, rows in ((_native.TILES_SHRINK, 48), (_native.TILES_EXPAND, 256)):
+        records, tile_rows = _native.plan_tiles(starts, ends, T, kind, r)
+        stray = torch.tensor([[1, 100, 100 + min(rows, tile_rows), 0], [2, 1290, 5000, 99]], dtype=torch.int32)
+        wrong = _native.TilePlan(torch.cat([torch.from_numpy(records.copy()), stray]).to(DEV), tile_rows)
+        good = _native.TilePlan(torch.from_numpy(records.copy()).to(DEV), tile_rows)
+        if kind == _native.TILES_SHRINK:
+            outs = []
+            previous = _native.set_fixed_order_shrink(True)  # two more tiles change the grid, and with it the order
+            try:                                             # of the sums, unless that order is fixed
+                for plan in (good, wrong):
+                    v = torch.zeros((T, r), dtype=dtype, device=DEV)
+                    _native.sgmv_shrink_multi([v], x, [ptr_table(a, DEV)], s_start, s_end, tmp, layer, 1.0, False, plan)
+                    outs.append(v)
+            finally:
+                _native.set_fixed_order_shrink(previous)
+        else:
+            vin = randn((T, r), 1.0, gen, dtype, DEV)
+            outs = []
+            for plan in (good, wrong):
+                y = torch.zeros((T, h_out), dtype=dtype, device=DEV)
+                _native.sgmv_expand(y, vin, ptr_table(bt, DEV), s_start, s_end, tmp_e, layer, 0, h_out, True, False, plan)
+                outs.append(y)
+        torch.cuda.synchronize()
+        # the stray tile over rows 1290.. of segment 2 is clamped to the batch and rewrites what its own tile wrote
+        differ = (outs[0] != outs[1]).nonzero()
+        assert differ.numel() == 0, f"kind {kind}: {differ.size(0)} elements differ, first {differ[:8].tolist()}"
+        assert torch.count_nonzero(outs[0]) > 0
