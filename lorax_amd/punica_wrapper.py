@@ -68,6 +68,7 @@ class PunicaWrapper:
         # to four tokens of one adapter, in a fixed buffer; _plan_records of them are in use
         self._plan = torch.zeros((max_num_batched_tokens, 8), dtype=torch.int64, device=device)
         self._plan_records: Optional[int] = None
+        self._plan_filled = 0  # records of the buffer that may be non-zero
 
     # ---- routing state ----------------------------------------------------------------------------
 
@@ -86,8 +87,11 @@ class PunicaWrapper:
             # run shrink and expand in one launch.
             if self._token_lora_indices.is_cuda and count <= self._plan.size(0):
                 records = ops.build_slot_plan(meta.adapter_indices.detach().cpu().numpy() - 1)
-                self._plan[: records.size(0)].copy_(records, non_blocking=True)
-                self._plan_records = records.size(0)
+                n, stale = records.size(0), self._plan_filled
+                self._plan[:n].copy_(records, non_blocking=True)
+                if stale > n:  # records of the batch before: all-zero records are padding the kernels skip, so a
+                    self._plan[n:stale].zero_()  # captured step that reads a fixed number of records stays right
+                self._plan_records = self._plan_filled = n
             return
         bounds = getattr(meta, "adapter_segments", None)
         owners = getattr(meta, "segment_indices", None)

@@ -253,3 +253,27 @@ def test_decode_with_a_slot_plan_equals_the_scanning_launches(dtype, ranks, widt
     wrapper.add_lora_slices(y_w, x, slices, 1.0)
     torch.cuda.synchronize()
     assert torch.equal(y_w, y_plan)
+
+
+def test_slot_plan_buffer_is_padded_with_skipped_records():
+    """The wrapper keeps its routing plan in one fixed buffer: after a smaller batch the records of the batch
+    before are zeroed, so a launch that reads a fixed number of records (a captured step) sees padding, which the
+    kernels skip, and gives the smaller batch's result."""
+    dtype, h_in, w, r, n = torch.bfloat16, 1024, 1024, 8, 5
+    gen = torch.Generator().manual_seed(3)
+    a, b = _stacks(n, r, h_in, w, gen, dtype)
+    wrapper = PunicaWrapper(128, 128, DEV, enabled=True)
+    big = torch.randint(0, n, (90,), generator=gen)
+    wrapper.update_metadata(make_meta((big + 1).tolist(), torch.device(DEV)), prefill=False)
+    first = wrapper._plan_records
+    small = torch.randint(-1, n, (23,), generator=gen)
+    wrapper.update_metadata(make_meta((small + 1).tolist(), torch.device(DEV)), prefill=False)
+    assert wrapper._plan_records < first
+    assert torch.count_nonzero(wrapper._plan[wrapper._plan_records:first]) == 0
+    x = randn((23, h_in), 1.0, gen, dtype, DEV)
+    y_fixed = torch.zeros((23, w), dtype=dtype, device=DEV)
+    ops.bgmv_lora_slices(x, [(a, b, 0, w)], y_fixed, small.to(DEV), 1.0, plan=wrapper._plan[:first])  # with the padding
+    y_ref = torch.zeros((23, w), dtype=dtype, device=DEV)
+    ops.bgmv_lora_slices(x, [(a, b, 0, w)], y_ref, small.to(DEV), 1.0)
+    torch.cuda.synchronize()
+    assert torch.equal(y_fixed, y_ref) and torch.count_nonzero(y_ref) > 0
